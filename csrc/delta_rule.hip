@@ -1,0 +1,240 @@
+// Gated delta-rule recurrence (prefill portions and single decode tokens in
+// one launch).
+//
+// Per head the state S is a D x D fp32 matrix (rows = key channels, columns
+// = value channels). For every token
+//     w = exp(-decay_scale * sigmoid(zw + w0))        per key channel
+//     a = sigmoid(za + ab)                            per key channel
+//     u = k / sqrt(sum(k^2) + 1e-6)
+//     S <- diag(w) S - (a*u)(u^T S) + k v^T           (both read the old S)
+//     o = S^T r
+// and the head's o is divided by its root mean square, scaled by a channel
+// weight and by sigmoid(g).
+//
+// Mapping: one workgroup per (sequence segment, head); thread j owns column
+// j of S in registers (DKP rows, D padded up), so u^T S and S^T r are
+// thread-local dot products and the only cross-lane traffic is the two
+// norms. Tokens go through in tiles: the per-row vectors (u, a*u, w, k, r)
+// of a whole tile are prepared cooperatively into LDS, then each thread
+// walks the tile's tokens with broadcast LDS reads and no barrier.
+#include "mix_common.h"
+
+template <typename T, int DKP, int TILE>
+__global__ __launch_bounds__(256) void delta_rule_kernel(
+    T* __restrict__ out, int ldo, const T* __restrict__ r, int ldr,
+    const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
+    const T* __restrict__ zw, int ldzw, const T* __restrict__ za, int ldza,
+    const T* __restrict__ g, int ldg, const float* __restrict__ w0,
+    const float* __restrict__ ab, const float* __restrict__ normw,
+    float* __restrict__ state, const int* __restrict__ seq_rows, int H, int D,
+    float eps, float decay_scale) {
+  extern __shared__ float lds[];
+  float* su = lds;                  // [TILE][DKP] unit key
+  float* sau = su + TILE * DKP;     // a * u
+  float* sw = sau + TILE * DKP;     // decay
+  float* sk = sw + TILE * DKP;      // key
+  float* sr = sk + TILE * DKP;      // receptance
+  float* red = sr + TILE * DKP;     // [4][TILE] cross-wave partials
+
+  const int seg = blockIdx.x / H, hd = blockIdx.x % H;
+  const int t0 = seq_rows[4 * seg + 0], n = seq_rows[4 * seg + 1];
+  const int p0 = seq_rows[4 * seg + 2], slot = seq_rows[4 * seg + 3];
+  const int j = threadIdx.x;
+  const bool col = j < D;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int hc = hd * D;  // channel offset of this head
+
+  float* Sg = state + ((size_t)slot * H + hd) * (size_t)D * D;
+  float S[DKP];
+#pragma unroll
+  for (int i = 0; i < DKP; ++i)
+    S[i] = (col && i < D && p0 != 0) ? Sg[(size_t)i * D + j] : 0.f;
+
+  for (int tb = 0; tb < n; tb += TILE) {
+    const int nt = min(TILE, n - tb);
+    __syncthreads();  // previous tile's LDS reads are done
+    for (int idx = threadIdx.x; idx < nt * DKP; idx += blockDim.x) {
+      const int tt = idx / DKP, i = idx % DKP;
+      float kv = 0.f, rv = 0.f, wv = 0.f, av = 0.f;
+      if (i < D) {
+        const size_t row = (size_t)(t0 + tb + tt);
+        const int c = hc + i;
+        kv = MxElem<T>::ld(k + row * ldk + c);
+        rv = MxElem<T>::ld(r + row * ldr + c);
+        const float z = MxElem<T>::ld(zw + row * ldzw + c) + w0[c];
+        wv = expf(-decay_scale * mx_sigmoid(z));
+        av = mx_sigmoid(MxElem<T>::ld(za + row * ldza + c) + ab[c]);
+      }
+      sk[idx] = kv;
+      sr[idx] = rv;
+      sw[idx] = wv;
+      sau[idx] = av;
+    }
+    __syncthreads();
+    for (int tt = wave; tt < nt; tt += nw) {
+      float ss = 0.f;
+      for (int i = lane; i < DKP; i += 64) {
+        const float kv = sk[tt * DKP + i];
+        ss += kv * kv;
+      }
+      ss = mx_wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss + 1e-6f);
+      for (int i = lane; i < DKP; i += 64) {
+        const float u = sk[tt * DKP + i] * inv;
+        su[tt * DKP + i] = u;
+        sau[tt * DKP + i] *= u;
+      }
+    }
+    __syncthreads();
+
+    float o[TILE];
+#pragma unroll
+    for (int tt = 0; tt < TILE; ++tt) {
+      o[tt] = 0.f;
+      if (tt < nt) {
+        const size_t row = (size_t)(t0 + tb + tt);
+        const float vj = col ? MxElem<T>::ld(v + row * ldv + hc + j) : 0.f;
+        const float* pu = su + tt * DKP;
+        const float* pau = sau + tt * DKP;
+        const float* pw = sw + tt * DKP;
+        const float* pk = sk + tt * DKP;
+        const float* pr = sr + tt * DKP;
+        float sa = 0.f;
+#pragma unroll
+        for (int i = 0; i < DKP; ++i) sa += pu[i] * S[i];
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < DKP; ++i) {
+          const float s = pw[i] * S[i] - pau[i] * sa + pk[i] * vj;
+          S[i] = s;
+          acc += s * pr[i];
+        }
+        o[tt] = acc;
+      }
+    }
+
+    // per-token sum over the head's columns of o^2
+#pragma unroll
+    for (int tt = 0; tt < TILE; ++tt) {
+      const float q = mx_wave_sum(col ? o[tt] * o[tt] : 0.f);
+      if (lane == 0) red[wave * TILE + tt] = q;
+    }
+    __syncthreads();
+    if (col) {
+#pragma unroll
+      for (int tt = 0; tt < TILE; ++tt) {
+        if (tt < nt) {
+          float ss = 0.f;
+          for (int w = 0; w < nw; ++w) ss += red[w * TILE + tt];
+          const size_t row = (size_t)(t0 + tb + tt);
+          const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+          const float gate =
+              mx_sigmoid(MxElem<T>::ld(g + row * ldg + hc + j));
+          MxElem<T>::st(out + row * ldo + hc + j,
+                        o[tt] * inv * normw[hc + j] * gate);
+        }
+      }
+    }
+  }
+  if (col) {
+#pragma unroll
+    for (int i = 0; i < DKP; ++i)
+      if (i < D) Sg[(size_t)i * D + j] = S[i];
+  }
+}
+
+template <typename T, int DKP>
+static void launch_delta(void* out, int ldo, const void* r, int ldr,
+                         const void* k, int ldk, const void* v, int ldv,
+                         const void* zw, int ldzw, const void* za, int ldza,
+                         const void* g, int ldg, const void* w0,
+                         const void* ab, const void* normw, void* state,
+                         const void* seq_rows, int S_, int H, int D,
+                         float eps, float decay_scale, hipStream_t stream) {
+  constexpr int TILE = DKP <= 128 ? 16 : 8;
+  const int threads = ((D + 63) / 64) * 64;
+  const size_t lds = (size_t)(5 * TILE * DKP + 4 * TILE) * sizeof(float);
+  hipLaunchKernelGGL((delta_rule_kernel<T, DKP, TILE>), dim3(S_ * H),
+                     dim3(threads), lds, stream, (T*)out, ldo, (const T*)r,
+                     ldr, (const T*)k, ldk, (const T*)v, ldv, (const T*)zw,
+                     ldzw, (const T*)za, ldza, (const T*)g, ldg,
+                     (const float*)w0, (const float*)ab,
+                     (const float*)normw, (float*)state,
+                     (const int*)seq_rows, H, D, eps, decay_scale);
+}
+
+#define DR_CASE(P)                                                          \
+  if (D <= P) {                                                             \
+    launch_delta<T, P>(out, ldo, r, ldr, k, ldk, v, ldv, zw, ldzw, za,      \
+                       ldza, g, ldg, w0, ab, normw, state, seq_rows, S_, H, \
+                       D, eps, decay_scale, (hipStream_t)stream);           \
+    return 0;                                                               \
+  }
+
+template <typename T>
+static int dispatch_delta(void* out, int ldo, const void* r, int ldr,
+                          const void* k, int ldk, const void* v, int ldv,
+                          const void* zw, int ldzw, const void* za, int ldza,
+                          const void* g, int ldg, const void* w0,
+                          const void* ab, const void* normw, void* state,
+                          const void* seq_rows, int S_, int H, int D,
+                          float eps, float decay_scale, void* stream) {
+  DR_CASE(16)
+  DR_CASE(32)
+  DR_CASE(48)
+  DR_CASE(64)
+  DR_CASE(80)
+  DR_CASE(96)
+  DR_CASE(112)
+  DR_CASE(128)
+  DR_CASE(192)
+  DR_CASE(256)
+  return 1;  // head dim above 256: not built
+}
+
+// The file may be compiled once per element type (MX_ONLY_DTYPE = 0 bf16,
+// 1 float) so the two sets of head-size instantiations build in parallel;
+// the float unit also carries the entry point.
+#define DR_ARGS                                                              \
+  void *out, int ldo, const void *r, int ldr, const void *k, int ldk,        \
+      const void *v, int ldv, const void *zw, int ldzw, const void *za,      \
+      int ldza, const void *g, int ldg, const void *w0, const void *ab,      \
+      const void *normw, void *state, const void *seq_rows, int S_, int H,   \
+      int D, float eps, float decay_scale, void *stream
+#define DR_PASS                                                              \
+  out, ldo, r, ldr, k, ldk, v, ldv, zw, ldzw, za, ldza, g, ldg, w0, ab,      \
+      normw, state, seq_rows, S_, H, D, eps, decay_scale, stream
+
+extern "C" int mx_delta_rule_bf16(DR_ARGS);
+extern "C" int mx_delta_rule_f32(DR_ARGS);
+
+#if !defined(MX_ONLY_DTYPE) || MX_ONLY_DTYPE == 0
+extern "C" int mx_delta_rule_bf16(DR_ARGS) {
+  return dispatch_delta<mx_bf16>(DR_PASS);
+}
+#endif
+#if !defined(MX_ONLY_DTYPE) || MX_ONLY_DTYPE == 1
+extern "C" int mx_delta_rule_f32(DR_ARGS) {
+  return dispatch_delta<float>(DR_PASS);
+}
+
+extern "C" int mx_delta_rule(void* out, int ldo, const void* r, int ldr,
+                             const void* k, int ldk, const void* v, int ldv,
+                             const void* zw, int ldzw, const void* za,
+                             int ldza, const void* g, int ldg,
+                             const void* w0, const void* ab,
+                             const void* normw, void* state,
+                             const void* seq_rows, int S_, int H, int D,
+                             float eps, float decay_scale, int dtype,
+                             void* stream) {
+  if (S_ <= 0) return 0;
+  if (dtype == MX_BF16)
+    return mx_delta_rule_bf16(out, ldo, r, ldr, k, ldk, v, ldv, zw, ldzw, za,
+                              ldza, g, ldg, w0, ab, normw, state, seq_rows,
+                              S_, H, D, eps, decay_scale, stream);
+  return mx_delta_rule_f32(out, ldo, r, ldr, k, ldk, v, ldv, zw, ldzw, za,
+                           ldza, g, ldg, w0, ab, normw, state, seq_rows, S_,
+                           H, D, eps, decay_scale, stream);
+}
+#endif

@@ -22,9 +22,20 @@ class BlockManager:
         num_blocks: int,
         block_size: int,
         enable_prefix_caching: bool = True,
+        num_state_slots: int = 0,
     ) -> None:
         self.num_blocks = num_blocks
         self.block_size = block_size
+        # per-sequence recurrent-state slots (models with recurrent
+        # layers): a live sequence owns one slot from admission until it
+        # is freed or preempted; the kernels zero a slot's state when a
+        # sequence's position 0 runs, so a reused slot needs no clearing.
+        # A recurrent state cannot be rebuilt from cached KV blocks, so
+        # prefix reuse is off for such models.
+        self.num_state_slots = num_state_slots
+        self.free_slots: deque[int] = deque(range(num_state_slots))
+        if num_state_slots:
+            enable_prefix_caching = False
         self.enable_prefix_caching = enable_prefix_caching
         self.free: deque[int] = deque(range(num_blocks))
         self.ref_count: List[int] = [0] * num_blocks
@@ -76,6 +87,8 @@ class BlockManager:
         return (num_tokens + self.block_size - 1) // self.block_size
 
     def can_allocate_prompt(self, seq: Sequence) -> bool:
+        if self.num_state_slots and not self.free_slots:
+            return False
         # worst case (no cache hits)
         return self.blocks_needed(seq.num_tokens) <= self.num_free
 
@@ -148,6 +161,12 @@ class BlockManager:
                 raise RuntimeError("out of KV blocks during prompt allocation")
             self.ref_count[blk] += 1
             table.append(blk)
+        if self.num_state_slots:
+            if not self.free_slots:
+                for b in table:
+                    self._release_block(b)
+                raise RuntimeError("out of recurrent-state slots")
+            seq.state_slot = self.free_slots.popleft()
         seq.block_table = table
         seq.num_cached_prompt_tokens = matched * bs
         seq.num_computed = matched * bs
@@ -213,6 +232,9 @@ class BlockManager:
         for blk in seq.block_table:
             self._release_block(blk)
         seq.block_table = []
+        if getattr(seq, "state_slot", None) is not None:
+            self.free_slots.append(seq.state_slot)
+            seq.state_slot = None
         self._tail_hash.pop(seq.request_id, None)
         if hasattr(seq, "_registered_full"):
             del seq._registered_full

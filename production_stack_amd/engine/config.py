@@ -16,6 +16,66 @@ from typing import Optional
 
 
 @dataclass
+class MixerSpec:
+    """One layer's token mixer.
+
+    kind "attention": softmax attention over a paged KV cache. `chunk`
+    restricts every query to keys of its own aligned block of positions
+    (0 = plain causal), `window` to the trailing N keys (0 = off), `sink`
+    adds a value-less key of score 0 to the softmax denominator,
+    `talking_heads` mixes the heads' scores with a learned [H, H] matrix
+    before the softmax, `rope` applies the rotary position code.
+    kind "general_delta": gated delta-rule linear recurrence with a
+    per-sequence fp32 state of heads x dim x dim; `decay_rank` is the
+    width of the low-rank decay projection.
+    """
+
+    kind: str
+    heads: int
+    dim: int
+    kv_heads: int = 0
+    vdim: int = 0
+    scale: float = 0.0
+    chunk: int = 0
+    window: int = 0
+    sink: bool = False
+    talking_heads: bool = False
+    rope: bool = True
+    decay_rank: int = 0
+
+
+@dataclass
+class MlpSpec:
+    """One layer's feed-forward. kind "dense": gated MLP with `act`.
+    kind "moe": `experts` small gated MLPs of width `ff`, `top` per token,
+    routed by `score` ("softmax" | "sigmoid") with optional renormalised
+    weights applied to the expert's output or (`weight_on_input`) input;
+    an always-on shared expert of width `shared_ff` may be added, scaled by
+    a per-token sigmoid gate."""
+
+    kind: str
+    ff: int
+    act: str = "silu"          # silu | gelu_tanh | clamped_swish
+    limit: float = 0.0
+    experts: int = 0
+    top: int = 0
+    score: str = "softmax"
+    renormalize: bool = True
+    weight_on_input: bool = False
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclass
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: Optional[MlpSpec]
+    # True: mixer and feed-forward both read one norm's output and their
+    # sum joins the residual; False: sequential pre-norm sublayers
+    parallel: bool = False
+
+
+@dataclass
 class ModelConfig:
     name: str
     hidden_size: int
@@ -42,6 +102,17 @@ class ModelConfig:
     # gate/up/down with per-expert projections + a top-k router
     num_experts: int = 0
     num_experts_per_tok: int = 2
+    # model family: selects the model class in engine/models/registry.py
+    family: str = "llama"
+    # heterogeneous stacks (family != "llama"): one spec per layer; the
+    # scalar head/ff fields above then hold the stack's maxima
+    layer_specs: Optional[list] = None
+    embedding_scale: float = 1.0
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return bool(self.layer_specs) and any(
+            ls.mixer.kind != "attention" for ls in self.layer_specs)
 
     @property
     def q_size(self) -> int:
@@ -397,6 +468,21 @@ class EngineConfig:
     parallel: ParallelConfig = field(default_factory=ParallelConfig)
 
     def model_config(self) -> ModelConfig:
+        import os
+
+        if os.path.isfile(os.path.join(self.model, "config.json")):
+            # a checkpoint folder: its config.json names the architecture
+            from production_stack_amd.engine.models.registry import (
+                config_from_dir,
+            )
+
+            cfg = config_from_dir(self.model)
+            if self.weights_path is None:
+                self.weights_path = self.model
+            if self.max_model_len > cfg.max_position:
+                cfg = dataclasses.replace(
+                    cfg, max_position=self.max_model_len)
+            return cfg
         if self.model not in ARCHITECTURES:
             raise ValueError(
                 f"unknown model architecture {self.model!r}; "

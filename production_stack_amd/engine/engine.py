@@ -61,6 +61,7 @@ class LLMEngine:
             num_blocks,
             config.cache.block_size,
             config.cache.enable_prefix_caching,
+            num_state_slots=self.runner.num_state_slots,
         )
         self.scheduler = Scheduler(
             config.scheduler, self.block_manager, config.max_model_len
@@ -134,6 +135,47 @@ class LLMEngine:
         self.scheduler.add(seq)
         self.stats.num_requests += 1
         self.stats.prompt_tokens += len(token_ids)
+
+    # ---- replay of given token streams (no sampling) ------------------
+    def replay_step(self, entries, end=()):
+        """Feed given tokens through the engine for one step and return
+        logits instead of sampling.
+
+        entries: [(request_id, tokens, want)], one per request taking part
+        in this step: its next tokens (a prompt portion or a single token)
+        and the offsets among them whose logits are wanted. A request is
+        admitted at its first entry, may sit out steps, and is freed
+        (blocks and state slot) once named in `end`. All entries run as
+        one batch through the scheduler's admission, the block manager and
+        the runner that generation uses. Returns fp32 logits
+        [sum(len(want)), vocab] in entry/want order (None when nothing is
+        wanted)."""
+        with self.lock:
+            plan = []
+            want = {}
+            for rid, tokens, offs in entries:
+                tokens = list(tokens)
+                if not tokens:
+                    continue
+                seq = self.scheduler.get(rid)
+                if seq is None:
+                    seq = Sequence(rid, tokens, SamplingParams(
+                        max_tokens=1, temperature=0.0, ignore_eos=True))
+                    self.scheduler.add(seq)
+                    self.stats.num_requests += 1
+                else:
+                    seq.prompt_token_ids.extend(tokens)
+                self.stats.prompt_tokens += len(tokens)
+                plan.append((seq, len(tokens)))
+                want[rid] = list(offs)
+            out = self.scheduler.schedule_plan(plan)
+            got = self.runner.execute_logits(out, self.block_manager, want)
+            self.scheduler.on_step_done(out, {}, self.model_cfg.eos_token_id)
+            for rid in end:
+                self.abort_request(rid)
+            parts = [got[rid] for rid, _, offs in entries
+                     if offs and rid in got]
+            return torch.cat(parts) if parts else None
 
     def abort_request(self, request_id: str) -> None:
         self.scheduler.abort(request_id)

@@ -15,7 +15,11 @@ import torch
 from production_stack_amd import ops
 from production_stack_amd.engine.block_manager import BlockManager
 from production_stack_amd.engine.config import EngineConfig, ModelConfig
-from production_stack_amd.engine.models.llama import BatchMeta, LlamaForCausalLM
+from production_stack_amd.engine.models.llama import BatchMeta
+from production_stack_amd.engine.models.registry import (
+    build_model,
+    load_weights,
+)
 from production_stack_amd.engine.scheduler import SchedulerOutput
 from production_stack_amd.engine.sequence import Sequence
 
@@ -38,9 +42,17 @@ class ModelRunner:
             import torch.distributed as dist
 
             self.pp_rank = dist.get_rank() if dist.is_initialized() else 0
-        self.model = LlamaForCausalLM(
-            model_cfg, tp=tp, pp_rank=self.pp_rank, pp_size=pp
+        self.model = build_model(
+            model_cfg, config.dtype, tp=tp, pp_rank=self.pp_rank, pp_size=pp
         ).to(device)
+        # heterogeneous stacks describe their per-layer cache themselves
+        # (paged KV for attention layers, per-sequence state for
+        # recurrent ones) and need whole-batch sequence metadata
+        self.hybrid = hasattr(self.model, "cache_shapes")
+        self.num_state_slots = (
+            config.scheduler.max_num_seqs
+            if model_cfg.has_recurrent_state else 0
+        )
         self.pipeline = None
         if pp > 1:
             from production_stack_amd.engine.pipeline import (
@@ -60,9 +72,7 @@ class ModelRunner:
             if dist.is_initialized():
                 self.tp_coord = TPCoordinator(self, ps.tp_rank(), tp)
         if config.weights_path:
-            from production_stack_amd.engine.weights import load_safetensors
-
-            load_safetensors(self.model, config.weights_path)
+            load_weights(self.model, config.weights_path)
         else:
             self.model.random_init(config.seed)
         self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
@@ -125,7 +135,11 @@ class ModelRunner:
             - (total - free)
         )
         per_block = self.model.kv_bytes_per_block(cache_cfg.block_size)
-        if self.kv_elem_bytes == 1:
+        if self.hybrid:
+            budget -= (self.num_state_slots
+                       * self.model.state_bytes_per_seq())
+            per_block = max(per_block, 1)
+        elif self.kv_elem_bytes == 1:
             per_block //= 2
         n = max(budget // per_block, 16)
         return int(n)
@@ -134,6 +148,29 @@ class ModelRunner:
         self.num_blocks = num_blocks
         cfg = self.model_cfg
         bs = self.config.cache.block_size
+        if self.hybrid:
+            # one entry per layer: (k, v) paged caches with the layer's own
+            # key/value widths, or the fp32 recurrent state [slots, heads,
+            # dim, vdim]
+            if self.config.cache.kv_cache_dtype not in ("auto", "bf16"):
+                raise ValueError(
+                    "this model family keeps its KV cache in the serving "
+                    "dtype (no fp8 KV)")
+            dt = self.model.dtype
+            self.kv_caches = []
+            for kind, heads, d, dv in self.model.cache_shapes():
+                if kind == "kv":
+                    self.kv_caches.append((
+                        torch.zeros((num_blocks, heads, bs, d), dtype=dt,
+                                    device=self.device),
+                        torch.zeros((num_blocks, heads, bs, dv), dtype=dt,
+                                    device=self.device),
+                    ))
+                else:
+                    self.kv_caches.append(torch.zeros(
+                        (max(self.num_state_slots, 1), heads, d, dv),
+                        dtype=torch.float32, device=self.device))
+            return
         kh = self.model.kv_heads
         kv_dt = self.config.cache.kv_cache_dtype
         dtype = (
@@ -161,6 +198,7 @@ class ModelRunner:
             # MoE routing is data-dependent (per-expert row gathers):
             # a captured decode graph would freeze one routing pattern
             or self.model_cfg.num_experts > 0
+            or not getattr(self.model, "supports_decode_graph", True)
         ):
             return
         from production_stack_amd.engine.graph_runner import DecodeGraphRunner
@@ -340,6 +378,33 @@ class ModelRunner:
             lora_idx_t = torch.full((row,), -1, dtype=torch.int32,
                                     device=dev)
 
+        seq_meta = {}
+        if getattr(self.model, "needs_seq_meta", False):
+            ordered = prefills + decodes
+            all_tabs = p_tables + d_tables
+            rows_np = np.zeros((len(ordered), 4), dtype=np.int32)
+            tok_seq = np.empty(len(tokens), dtype=np.int32)
+            r0 = 0
+            for i, ss in enumerate(ordered):
+                slot = ss.seq.state_slot
+                if self.num_state_slots and not (
+                        slot is not None
+                        and 0 <= slot < self.num_state_slots):
+                    raise RuntimeError(
+                        f"sequence {ss.seq.request_id} has no valid "
+                        "recurrent-state slot")
+                rows_np[i] = (r0, ss.num_tokens, ss.seq.num_computed,
+                              slot or 0)
+                tok_seq[r0:r0 + ss.num_tokens] = i
+                r0 += ss.num_tokens
+            seq_meta = dict(
+                block_tables=pad_tables(all_tabs),
+                token_seq=torch.from_numpy(tok_seq).to(
+                    dev, non_blocking=True),
+                seq_rows=torch.from_numpy(rows_np).to(
+                    dev, non_blocking=True),
+            )
+
         meta = BatchMeta(
             positions=torch.tensor(positions, dtype=torch.int32).to(
                 dev, non_blocking=True
@@ -393,6 +458,7 @@ class ModelRunner:
                 if mm_parts
                 else None
             ),
+            **seq_meta,
         )
         token_t = torch.tensor(tokens, dtype=torch.long).to(
             dev, non_blocking=True
@@ -558,6 +624,45 @@ class ModelRunner:
             out, sample_seqs, logits, self.sample(logits, sample_seqs)
         )
         return self._collect_sampled(out, sample_seqs, tokens, logits)
+
+    @torch.no_grad()
+    def execute_logits(
+        self, out: SchedulerOutput, bm: BlockManager,
+        want: Dict[str, List[int]],
+    ) -> Dict[str, torch.Tensor]:
+        """Run one step without sampling and return fp32 logits at chosen
+        places: want maps request_id -> offsets into that request's chunk
+        of this step. Same batch preparation, model forward and caches as
+        execute(); used to replay given token streams (scoring)."""
+        token_t, meta, _, _ = self.prepare(out, bm)
+        if token_t.numel() == 0:
+            return {}
+        if self.pipeline is not None or self.tp_coord is not None:
+            raise NotImplementedError("logit replay runs on one GPU")
+        hidden = self.model(token_t, meta, self.kv_caches)
+        # batch layout: multi-token chunks first, then single tokens
+        ordered = ([s for s in out.scheduled if not s.is_decode]
+                   + [s for s in out.scheduled if s.is_decode])
+        rows: List[int] = []
+        spans: Dict[str, tuple] = {}
+        r0 = 0
+        for ss in ordered:
+            offs = want.get(ss.seq.request_id) or []
+            for o in offs:
+                if not 0 <= o < ss.num_tokens:
+                    raise IndexError(
+                        f"wanted offset {o} outside the {ss.num_tokens}-"
+                        f"token chunk of {ss.seq.request_id}")
+            spans[ss.seq.request_id] = (len(rows), len(offs))
+            rows.extend(r0 + o for o in offs)
+            r0 += ss.num_tokens
+        if not rows:
+            return {}
+        rows_t = torch.tensor(rows, dtype=torch.long,
+                              device=hidden.device)
+        logits = self.model.compute_logits(
+            hidden.index_select(0, rows_t)).float()
+        return {rid: logits[a:a + n] for rid, (a, n) in spans.items() if n}
 
     @torch.no_grad()
     def _execute_pp_microbatched(

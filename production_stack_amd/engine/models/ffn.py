@@ -1,0 +1,166 @@
+"""Feed-forward building blocks shared by the model families.
+
+  * route():       fp32 router with softmax or sigmoid scores, top-k and
+                   optional renormalisation of the chosen weights;
+  * sparse_moe():  expert dispatch: rows are sorted by expert once (one
+                   host read of the per-expert counts per call) and every
+                   expert runs the dense GEMM path over its slice, with the
+                   routing weight on the expert's output or on its input;
+  * GatedMLP / SparseMoE: parameter holders driven by engine.config.MlpSpec,
+                   used by the heterogeneous (per-layer spec) models.
+
+The Llama family's Mixtral layers call route()/sparse_moe() too.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from production_stack_amd import ops
+from production_stack_amd.engine.config import MlpSpec
+from production_stack_amd.ops import gemm_policy
+
+
+def route(x: torch.Tensor, router_w: torch.Tensor, top: int,
+          score: str = "softmax", renormalize: bool = True):
+    """Returns (weights fp32 [T, top], expert ids [T, top]). The logits are
+    an fp32 product of the (up-cast) activations and router weights."""
+    logits = F.linear(x.float(), router_w.float())
+    if score == "softmax":
+        probs = torch.softmax(logits, dim=-1)
+    elif score == "sigmoid":
+        probs = torch.sigmoid(logits)
+    else:
+        raise ValueError(f"unknown router score {score!r}")
+    weights, sel = torch.topk(probs, top, dim=-1)
+    if renormalize:
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    return weights, sel
+
+
+def sparse_moe(x: torch.Tensor, weights: torch.Tensor, sel: torch.Tensor,
+               n_experts: int,
+               expert_fn: Callable[[int, torch.Tensor], torch.Tensor],
+               weight_on_input: bool = False,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sum over chosen experts of  w * expert(x)  (or expert(w * x)).
+
+    expert_fn(e, rows_of_x) -> rows_of_y. `out` (zero-filled [T, width],
+    any float dtype) is accumulated into and returned; it defaults to x's
+    dtype."""
+    T, K = sel.shape
+    if out is None:
+        out = torch.zeros_like(x)
+    flat = sel.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=n_experts).tolist()
+    rows_sorted = torch.div(order, K, rounding_mode="floor")
+    w_sorted = weights.reshape(-1)[order]
+    start = 0
+    for e, n in enumerate(counts):
+        if n == 0:
+            continue
+        rows = rows_sorted[start:start + n]
+        w = w_sorted[start:start + n]
+        start += n
+        xe = x.index_select(0, rows)
+        if weight_on_input:
+            xe = (xe.float() * w.unsqueeze(-1)).to(x.dtype)
+            ye = expert_fn(e, xe)
+        else:
+            ye = expert_fn(e, xe) * w.to(x.dtype).unsqueeze(-1)
+        out.index_add_(0, rows, ye.to(out.dtype))
+    return out
+
+
+class GatedMLP(nn.Module):
+    """down(act(gate x) * up x); gate and up are one fused projection. The
+    fused in-projection may be run by the caller together with other
+    consumers of the same input (see in_params / forward_from_proj)."""
+
+    def __init__(self, width: int, ff: int, act: str, limit: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.ff, self.act, self.limit = ff, act, limit
+        self.gate_up = nn.Parameter(torch.empty(2 * ff, width, dtype=dtype))
+        self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype))
+
+    def in_params(self):
+        return [self.gate_up]
+
+    def inner(self, proj: torch.Tensor,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """proj [T, 2*ff] = gate | up  ->  activation [T, ff]."""
+        return ops.gated_act(proj[:, :self.ff], proj[:, self.ff:], self.act,
+                             self.limit, out=out)
+
+    def forward_from_proj(self, proj: torch.Tensor) -> torch.Tensor:
+        return gemm_policy.linear(self.inner(proj), self.down)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.forward_from_proj(gemm_policy.linear(x, self.gate_up))
+
+
+class SparseMoE(nn.Module):
+    """Routed experts (+ optional always-on shared expert scaled by a
+    per-token sigmoid gate), configured by an MlpSpec."""
+
+    def __init__(self, width: int, spec: MlpSpec, dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec = spec
+        E, ff = spec.experts, spec.ff
+        self.router = nn.Parameter(torch.empty(E, width, dtype=dtype))
+        self.experts_gate_up = nn.Parameter(
+            torch.empty(E, 2 * ff, width, dtype=dtype))
+        self.experts_down = nn.Parameter(
+            torch.empty(E, width, ff, dtype=dtype))
+        self.shared = None
+        if spec.shared_ff:
+            self.shared = GatedMLP(width, spec.shared_ff, spec.act,
+                                   spec.shared_limit, dtype)
+            self.shared_gate = nn.Parameter(
+                torch.empty(1, width, dtype=dtype))
+
+    def in_params(self):
+        """Parameters the caller may fold into a fused projection of the
+        layer input: shared gate|up, then the shared expert's scalar
+        gate."""
+        if self.shared is None:
+            return []
+        return [self.shared.gate_up, self.shared_gate]
+
+    def _expert(self, e: int, xe: torch.Tensor) -> torch.Tensor:
+        ff = self.spec.ff
+        gu = gemm_policy.linear(xe, self.experts_gate_up[e])
+        act = ops.gated_act(gu[:, :ff], gu[:, ff:], self.spec.act,
+                            self.spec.limit)
+        return gemm_policy.linear(act, self.experts_down[e])
+
+    def forward_from_proj(self, x: torch.Tensor,
+                          proj: Optional[torch.Tensor]) -> torch.Tensor:
+        """x: layer input [T, width]; proj: the shared expert's fused
+        projection [T, 2*shared_ff + 1] (None without a shared expert).
+        Returns fp32 [T, width]: several experts' outputs are summed in
+        fp32."""
+        sp = self.spec
+        weights, sel = route(x, self.router, sp.top, sp.score,
+                             sp.renormalize)
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        sparse_moe(x, weights, sel, sp.experts, self._expert,
+                   weight_on_input=sp.weight_on_input, out=out)
+        if self.shared is not None:
+            sff = sp.shared_ff
+            y = self.shared.forward_from_proj(proj[:, :2 * sff])
+            gate = torch.sigmoid(proj[:, 2 * sff:].float())
+            out += y.float() * gate
+        return out
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        ps = self.in_params()
+        proj = (gemm_policy.linear(x, torch.cat(list(ps), dim=0))
+                if ps else None)
+        return self.forward_from_proj(x, proj)

@@ -86,6 +86,42 @@ class Scheduler:
         self._by_id[seq.request_id] = seq
         self.waiting.append(seq)
 
+    def get(self, request_id: str) -> Optional[Sequence]:
+        return self._by_id.get(request_id)
+
+    def schedule_plan(self, plan) -> SchedulerOutput:
+        """Externally planned step: plan = [(sequence, tokens to run)].
+        Waiting sequences are admitted and running ones grown through the
+        same block-manager calls as schedule(); nothing is preempted — a
+        plan that does not fit the cache or the sequence slots is an
+        error of the caller."""
+        out = SchedulerOutput()
+        for seq, n in plan:
+            if seq.status is SeqStatus.WAITING:
+                if len(self.running) >= self.config.max_num_seqs:
+                    raise RuntimeError(
+                        f"plan admits {seq.request_id} beyond max_num_seqs "
+                        f"{self.config.max_num_seqs}")
+                if not self.bm.can_allocate_prompt(seq):
+                    raise RuntimeError(
+                        f"no cache room to admit {seq.request_id}")
+                self.waiting.remove(seq)
+                self.bm.allocate_prompt(seq)
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+            elif seq.status is not SeqStatus.RUNNING:
+                raise RuntimeError(
+                    f"{seq.request_id} is {seq.status.value}, not runnable")
+            if n < 1 or seq.num_computed + n > seq.num_tokens:
+                raise ValueError(
+                    f"plan runs {n} tokens of {seq.request_id} but "
+                    f"{seq.num_tokens - seq.num_computed} are pending")
+            if not self.bm.ensure_capacity(seq, seq.num_computed + n):
+                raise RuntimeError(
+                    f"KV cache exhausted growing {seq.request_id}")
+            out.scheduled.append(ScheduledSeq(seq, n))
+        return out
+
     def abort(self, request_id: str) -> Optional[Sequence]:
         seq = self._by_id.pop(request_id, None)
         if seq is None or seq.finished:

@@ -54,6 +54,9 @@ class Sequence:
         self.num_computed = 0  # tokens with KV in cache and attended
         self._draft_progress = 0  # draft-model KV progress (engine/draft.py)
         self.block_table: List[int] = []
+        # recurrent-state slot (models with recurrent layers), owned from
+        # admission to free/preemption; None otherwise
+        self.state_slot: Optional[int] = None
         self.num_cached_prompt_tokens = 0  # prefix-cache hits at admission
         # streaming cursor: outputs not yet handed to the consumer
         self._stream_cursor = 0

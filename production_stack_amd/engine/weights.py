@@ -15,6 +15,20 @@ import torch
 from production_stack_amd.parallel import state as pstate
 
 
+def safetensors_header(path: str) -> dict:
+    """name -> {dtype, shape, data_offsets} of a .safetensors file (an
+    8-byte little-endian length, then that many bytes of JSON), without
+    touching the tensor data."""
+    import json
+    import struct
+
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        head = json.loads(f.read(n))
+    head.pop("__metadata__", None)
+    return head
+
+
 def load_safetensors(model, path: str) -> None:
     from safetensors.torch import load_file
 

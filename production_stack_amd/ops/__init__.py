@@ -407,3 +407,216 @@ def fp8_linear_rowwise(xq, sx, w_q, sw):
     out = torch._scaled_mm(xq, w_q.t(), scale_a=one, scale_b=one,
                            out_dtype=torch.float32)
     return (out * sx[:, None] * sw[None, :]).to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------
+# fp32-residual stack ops (hybrid recurrent/attention models). On a GPU
+# these run the kernels of `_mixops.so` (ops/native.py) for bf16 or float32
+# activations; on CPU tensors the references run.
+# ---------------------------------------------------------------------------
+ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2}
+
+
+def _mx():
+    from production_stack_amd.ops import native
+
+    return native.load()
+
+
+def _mx_dtype(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return 0
+    if dtype == torch.float32:
+        return 1
+    raise TypeError(f"mixer kernels take bfloat16 or float32, not {dtype}")
+
+
+def _stream():
+    import ctypes
+
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    import ctypes
+
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """Row stride (elements) of a 2-D view whose rows are contiguous."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name}: need a 2-D view with unit inner stride")
+    return t.stride(0)
+
+
+def embed_scale(tokens: torch.Tensor, embed: torch.Tensor,
+                scale: float) -> torch.Tensor:
+    """fp32 residual rows embed[token] * scale."""
+    if not embed.is_cuda:
+        return reference.embed_scale(tokens, embed, scale)
+    T, W = tokens.shape[0], embed.shape[1]
+    assert tokens.dtype == torch.long and tokens.is_contiguous()
+    assert embed.is_contiguous()
+    x = torch.empty((T, W), dtype=torch.float32, device=embed.device)
+    _mx().mx_embed_scale(_p(x), _p(tokens), _p(embed),
+                         _f(scale), T, W, _mx_dtype(embed.dtype), _stream())
+    return x
+
+
+def _f(v: float):
+    import ctypes
+
+    return ctypes.c_float(v)
+
+
+def add_rms_norm32(x32: torch.Tensor, deltas, w32: torch.Tensor, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """x32 += sum(deltas) (fp32, in place; up to two deltas of out_dtype),
+    returns rms_norm(x32) * w32 rounded to out_dtype."""
+    if not x32.is_cuda:
+        return reference.add_rms_norm32(x32, deltas, w32, eps, out_dtype)
+    T, W = x32.shape
+    assert x32.dtype == torch.float32 and x32.is_contiguous()
+    assert w32.dtype == torch.float32 and w32.numel() == W
+    deltas = list(deltas)
+    if len(deltas) > 2:
+        raise ValueError("at most two deltas")
+    for d in deltas:
+        assert d.dtype == out_dtype and d.shape == (T, W)
+    d0 = deltas[0] if deltas else None
+    d1 = deltas[1] if len(deltas) > 1 else None
+    h = torch.empty((T, W), dtype=out_dtype, device=x32.device)
+    _mx().mx_add_rms_norm32(
+        _p(h), _p(x32), _p(d0), _rows(d0, "delta") if d0 is not None else 0,
+        _p(d1), _rows(d1, "delta") if d1 is not None else 0, _p(w32),
+        _f(eps), T, W, _mx_dtype(out_dtype), _stream())
+    return h
+
+
+def gated_act(gate: torch.Tensor, up: torch.Tensor, kind: str,
+              limit: float = 0.0, out: torch.Tensor = None) -> torch.Tensor:
+    """Gated-MLP inner activation on [T, F] views (row-strided allowed):
+    silu | gelu_tanh | clamped_swish (see reference.gated_act)."""
+    T, F = gate.shape
+    assert up.shape == (T, F) and up.dtype == gate.dtype
+    if out is None:
+        out = torch.empty((T, F), dtype=gate.dtype, device=gate.device)
+    assert out.shape == (T, F) and out.dtype == gate.dtype
+    if not gate.is_cuda:
+        out.copy_(reference.gated_act(gate, up, kind, limit, gate.dtype))
+        return out
+    _mx().mx_gated_act(
+        _p(out), _rows(out, "out"), _p(gate), _rows(gate, "gate"), _p(up),
+        _rows(up, "up"), T, F, ACT_KINDS[kind], _f(limit),
+        _mx_dtype(gate.dtype), _stream())
+    return out
+
+
+def kv_append(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+              v_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """Append k [T, G*D] / v [T, G*DV] rows (row-strided views allowed) to
+    paged caches [NB, G, BS, D] / [NB, G, BS, DV]."""
+    NB, G, BS, D = k_cache.shape
+    DV = v_cache.shape[3]
+    T = k.shape[0]
+    assert v_cache.shape[:3] == (NB, G, BS)
+    assert k.shape == (T, G * D) and v.shape == (T, G * DV)
+    assert slot_mapping.dtype == torch.long and slot_mapping.shape == (T,)
+    if not k_cache.is_cuda:
+        reference.kv_append(k.reshape(T, G, D), v.reshape(T, G, DV),
+                            k_cache, v_cache, slot_mapping)
+        return
+    assert k.dtype == k_cache.dtype == v.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    _mx().mx_kv_append(
+        _p(k), _rows(k, "k"), _p(v), _rows(v, "v"), _p(k_cache),
+        _p(v_cache), _p(slot_mapping), T, G, D, DV, BS,
+        _mx_dtype(k.dtype), _stream())
+
+
+def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
+                   v_cache: torch.Tensor, block_tables: torch.Tensor,
+                   token_seq: torch.Tensor, token_pos: torch.Tensor,
+                   scale: float, heads: int, chunk: int = 0, window: int = 0,
+                   sink: bool = False, talk: torch.Tensor = None,
+                   out: torch.Tensor = None) -> torch.Tensor:
+    """Paged attention of a ragged batch. q [T, H*D] (row-strided view
+    allowed); token_seq/token_pos int32 [T] give each token's block-table
+    row and position; talk: optional fp32 [H, H] score mix; chunk/window:
+    visibility limits (0 = off); sink: add 1 to the softmax denominator.
+    Returns [T, H*DV]."""
+    NB, G, BS, D = k_cache.shape
+    DV = v_cache.shape[3]
+    T = q.shape[0]
+    H = heads
+    assert q.shape == (T, H * D) and H % G == 0
+    assert token_seq.dtype == torch.int32 and token_pos.dtype == torch.int32
+    assert token_seq.shape == (T,) and token_pos.shape == (T,)
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2
+    if talk is not None:
+        assert talk.dtype == torch.float32 and talk.shape == (H, H)
+    if out is None:
+        out = torch.empty((T, H * DV), dtype=q.dtype, device=q.device)
+    assert out.shape == (T, H * DV) and out.dtype == q.dtype
+    if not q.is_cuda:
+        o = reference.talk_attention(
+            q.reshape(T, H, D), k_cache, v_cache, block_tables, token_seq,
+            token_pos, scale, chunk, window, sink, talk)
+        out.copy_(o.reshape(T, H * DV))
+        return out
+    assert q.dtype == k_cache.dtype == v_cache.dtype
+    assert block_tables.is_contiguous()
+    if talk is not None:
+        assert talk.is_contiguous()
+    rc = _mx().mx_talk_attention(
+        _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
+        _p(v_cache), _p(block_tables), block_tables.shape[1],
+        _p(token_seq), _p(token_pos), _p(talk), T, H, G, D, DV, BS,
+        _f(scale), int(chunk), int(window), int(bool(sink)),
+        _mx_dtype(q.dtype), _stream())
+    if rc != 0:
+        raise RuntimeError(
+            f"talk_attention: heads x dim {H}x{D}/{DV} exceeds the kernel's "
+            "LDS budget")
+    return out
+
+
+def delta_rule(r, k, v, zw, za, g, w0, ab, normw, state, seq_rows,
+               heads: int, eps: float, decay_scale: float,
+               out: torch.Tensor = None) -> torch.Tensor:
+    """Gated delta-rule recurrence over a ragged batch (see
+    reference.delta_rule). r/k/v/zw/za/g: [T, H*D] row-strided views of one
+    dtype; w0/ab/normw fp32 [H*D]; state fp32 [slots, H, D, D], updated in
+    place; seq_rows int32 [S, 4] = (first row, rows, first position, state
+    slot) per segment. Returns [T, H*D] (written into `out` when given)."""
+    T, HD = r.shape
+    H = heads
+    D = HD // H
+    assert state.dtype == torch.float32 and state.shape[1:] == (H, D, D)
+    assert seq_rows.dtype == torch.int32 and seq_rows.shape[1] == 4
+    for name, t in (("k", k), ("v", v), ("zw", zw), ("za", za), ("g", g)):
+        assert t.shape == (T, HD) and t.dtype == r.dtype, name
+    for t in (w0, ab, normw):
+        assert t.dtype == torch.float32 and t.numel() == HD
+    if out is None:
+        out = torch.empty((T, HD), dtype=r.dtype, device=r.device)
+    assert out.shape == (T, HD) and out.dtype == r.dtype
+    if not r.is_cuda:
+        sh = (T, H, D)
+        y = reference.delta_rule(
+            r.reshape(sh), k.reshape(sh), v.reshape(sh), zw.reshape(sh),
+            za.reshape(sh), g.reshape(sh), w0, ab, normw, state, seq_rows,
+            eps, decay_scale, r.dtype)
+        out.copy_(y.reshape(T, HD))
+        return out
+    assert state.is_contiguous() and seq_rows.is_contiguous()
+    rc = _mx().mx_delta_rule(
+        _p(out), _rows(out, "out"), _p(r), _rows(r, "r"), _p(k),
+        _rows(k, "k"), _p(v), _rows(v, "v"), _p(zw), _rows(zw, "zw"),
+        _p(za), _rows(za, "za"), _p(g), _rows(g, "g"), _p(w0), _p(ab),
+        _p(normw), _p(state), _p(seq_rows), seq_rows.shape[0], H, D,
+        _f(eps), _f(decay_scale), _mx_dtype(r.dtype), _stream())
+    if rc != 0:
+        raise RuntimeError(f"delta_rule: head dim {D} above 256 is not built")
+    return out

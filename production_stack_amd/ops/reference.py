@@ -200,3 +200,129 @@ def lora_bgmv(out, x, A, B, scale, idx, col_off):
             continue
         y = (A[s].float() @ x[t].float()) * float(scale[s])
         out[t, col_off : col_off + W] += (B[s].float() @ y).to(out.dtype)
+
+
+# ---------------------------------------------------------------------------
+# fp32-residual stack ops (hybrid recurrent/attention models)
+# ---------------------------------------------------------------------------
+def embed_scale(tokens, embed, scale: float) -> torch.Tensor:
+    """fp32 residual stream rows: embed[token] * scale."""
+    return embed[tokens].float() * scale
+
+
+def add_rms_norm32(x32, deltas, w32, eps: float, out_dtype):
+    """x32 += sum(deltas) in fp32 (in place); returns norm(x32) * w32 in
+    out_dtype."""
+    if deltas:
+        acc = deltas[0].float()
+        for d in deltas[1:]:
+            acc = acc + d.float()
+        x32 += acc
+    var = x32.pow(2).mean(dim=-1, keepdim=True)
+    return (x32 * torch.rsqrt(var + eps) * w32).to(out_dtype)
+
+
+def gated_act(gate, up, kind: str, limit: float, out_dtype):
+    """Gated-MLP inner activation, fp32 math, one rounding at the end.
+    silu: silu(g)*u; gelu_tanh: gelu_tanh(g)*u; clamped_swish:
+    g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(1.702 g') (u'+1).
+    """
+    g = gate.float()
+    u = up.float()
+    if kind == "silu":
+        y = torch.nn.functional.silu(g) * u
+    elif kind == "gelu_tanh":
+        y = torch.nn.functional.gelu(g, approximate="tanh") * u
+    elif kind == "clamped_swish":
+        g = torch.clamp(g, max=limit)
+        u = torch.clamp(u, min=-limit, max=limit)
+        y = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+    else:
+        raise ValueError(kind)
+    return y.to(out_dtype)
+
+
+def kv_append(k, v, k_cache, v_cache, slot_mapping) -> None:
+    """k [T, G, D], v [T, G, DV] -> caches [NB, G, BS, D|DV] (k and v may
+    differ in their last dim)."""
+    bs = k_cache.shape[2]
+    blk = (slot_mapping // bs).long()
+    off = (slot_mapping % bs).long()
+    k_cache[blk, :, off] = k.to(k_cache.dtype)
+    v_cache[blk, :, off] = v.to(v_cache.dtype)
+
+
+def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
+                   scale: float, chunk: int, window: int, sink: bool,
+                   talk):
+    """Paged attention with optional head-mixed scores, aligned-chunk or
+    trailing-window visibility and a denominator sink. q [T, H, D];
+    returns [T, H, DV] in q's dtype; all score math in fp32."""
+    T, H, D = q.shape
+    G, bs, DV = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    out = torch.zeros(T, H, DV, dtype=torch.float32)
+    tk = talk.float() if talk is not None else None
+    for t in range(T):
+        pos = int(token_pos[t])
+        lo = 0
+        if chunk > 0:
+            lo = (pos // chunk) * chunk
+        if window > 0:
+            lo = max(lo, pos - window + 1)
+        idx = torch.arange(lo, pos + 1)
+        table = block_tables[int(token_seq[t])].long()
+        blk = table[idx // bs]
+        off = idx % bs
+        kk = k_cache[blk, :, off].float()          # [n, G, D]
+        vv = v_cache[blk, :, off].float()          # [n, G, DV]
+        kk = kk.repeat_interleave(rep, dim=1)      # [n, H, D]
+        vv = vv.repeat_interleave(rep, dim=1)
+        s = torch.einsum("hd,nhd->hn", q[t].float(), kk) * scale
+        if tk is not None:
+            s = tk @ s
+        m = s.max(dim=-1, keepdim=True).values
+        if sink:
+            m = torch.clamp(m, min=0.0)
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True)
+        if sink:
+            den = den + torch.exp(-m)
+        out[t] = torch.einsum("hn,nhv->hv", e / den, vv)
+    return out.to(q.dtype)
+
+
+def delta_rule(r, k, v, zw, za, g, w0, ab, normw, state, seq_rows,
+               eps: float, decay_scale: float, out_dtype):
+    """Gated delta-rule recurrence over a ragged batch.
+
+    r/k/v/zw/za/g: [T, H, D] views (any float dtype); w0/ab/normw fp32
+    [H*D]; state fp32 [slots, H, D, D] updated in place; seq_rows
+    [S, 4] int (first row, rows, first position, state slot). Per token
+      w = exp(-decay_scale * sigmoid(zw + w0)),  a = sigmoid(za + ab),
+      u = k / sqrt(sum k^2 + 1e-6),
+      S <- diag(w) S - (a*u)(u^T S) + k v^T,   o = S^T r,
+    then o / rms(o) per head * normw * sigmoid(g). A segment whose first
+    position is 0 starts from a zero state."""
+    T, H, D = r.shape
+    out = torch.empty(T, H, D, dtype=torch.float32)
+    w0 = w0.view(H, D)
+    ab = ab.view(H, D)
+    for t0, n, p0, slot in seq_rows.tolist():
+        S = state[slot]
+        if p0 == 0:
+            S.zero_()
+        for t in range(t0, t0 + n):
+            kk = k[t].float()
+            w = torch.exp(-decay_scale * torch.sigmoid(zw[t].float() + w0))
+            a = torch.sigmoid(za[t].float() + ab)
+            u = kk * torch.rsqrt((kk * kk).sum(-1, keepdim=True) + 1e-6)
+            sa = torch.einsum("hi,hij->hj", u, S)
+            S.mul_(w.unsqueeze(-1))
+            S.sub_((a * u).unsqueeze(-1) * sa.unsqueeze(1))
+            S.add_(kk.unsqueeze(-1) * v[t].float().unsqueeze(1))
+            out[t] = torch.einsum("hij,hi->hj", S, r[t].float())
+    var = out.pow(2).mean(-1, keepdim=True)
+    y = out * torch.rsqrt(var + eps) * normw.view(1, H, D)
+    y = y * torch.sigmoid(g.float())
+    return y.to(out_dtype)

@@ -46,6 +46,8 @@ ext = CUDAExtension(
             "-O3",
             "-std=c++17",
             "--offload-arch=gfx950",
+            # packed-fp32 instruction forms stay off for every HIP file
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         ],
     },
 )
