@@ -323,8 +323,11 @@ class ModelRunner:
             slots.append(seq.block_table[pos // bs] * bs + pos % bs)
             d_seq_lens.append(pos + 1)
             d_tables.append(seq.block_table)
-            sample_rows.append(len(tokens) - 1)
-            sample_seqs.append(seq)
+            # a one-token chunk in the middle of a prompt (the step's
+            # token budget ran out) is not a decode: nothing is sampled
+            if pos + 1 == seq.num_tokens:
+                sample_rows.append(len(tokens) - 1)
+                sample_seqs.append(seq)
 
         max_bt = max((len(t) for t in p_tables + d_tables), default=1)
 
@@ -485,6 +488,9 @@ class ModelRunner:
             or n == 0
             or self.graphs.bucket_for(n) is None
             or any(not s.is_decode for s in scheduled)
+            # one-token chunks inside a prompt sample nothing: eager path
+            or any(s.seq.num_computed + 1 != s.seq.num_tokens
+                   for s in scheduled)
             or (self.lora_slots is None
                 and any(s.seq.lora_name for s in scheduled))
         ):

@@ -721,3 +721,14 @@ def test_prompt_logprobs_chunking_invariant():
     assert got2 is not None
     for a, b in zip(one[1:], got2[1:]):
         assert abs(a - b) < 1e-3, (a, b)
+
+
+def test_one_token_prompt_chunk_samples_nothing():
+    """A token budget that leaves ONE token for a prompt in the middle of
+    its prefill must not be taken for a decode step: nothing is sampled
+    until the prompt's last token has run."""
+    prompts = [list(range(10, 55)), [7, 8, 9], list(range(100, 128))]
+    p = SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True)
+    big = make_engine(max_num_batched_tokens=256).generate(prompts, p)
+    small = make_engine(max_num_batched_tokens=7).generate(prompts, p)
+    assert big == small

@@ -1,0 +1,419 @@
+"""Each Nanurax mechanism alone: the engine's building blocks (ops + the
+mixer / feed-forward modules, with their paged cache and state slots) against
+the float64 oracle in tests/oracle_nanurax.py. CPU runs the reference ops,
+the gpu-marked variants run the HIP kernels."""
+
+import math
+
+import pytest
+import torch
+
+import oracle_nanurax as O
+from nanurax_util import (TOL, attn, delta, make_cfg, make_weights, moe,
+                          rel_err)
+from production_stack_amd.engine.config import MlpSpec
+from production_stack_amd.engine.models import nanurax as nx
+from production_stack_amd.engine.models.ffn import GatedMLP, SparseMoE
+from production_stack_amd.engine.models.llama import BatchMeta
+from production_stack_amd.engine.models.mixers import build_mixer
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DTYPES = ["float32", "bfloat16"]
+TD = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+pytestmark = pytest.mark.filterwarnings("ignore::UserWarning")
+
+
+def rnd(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------
+# feed-forwards
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_dense_feed_forward(device, dtype):
+    width, ff = 40, 72
+    W = {"gate": rnd((ff, width), 1, 0.3), "up": rnd((ff, width), 2, 0.3),
+         "down": rnd((width, ff), 3, 0.2)}
+    h = rnd((13, width), 4, 1.5)
+    want = O.dense_ff(h, W["gate"], W["up"], W["down"])
+    m = GatedMLP(width, ff, "gelu_tanh", 0.0, TD[dtype])
+    with torch.no_grad():
+        m.gate_up.copy_(torch.cat([W["gate"], W["up"]]))
+        m.down.copy_(W["down"])
+    m = m.to(device)
+    got = m(h.to(TD[dtype]).to(device))
+    assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("top,shared", [(1, None), (2, (24, 0.75)),
+                                        (3, (16, 3.0))])
+def test_routed_feed_forward(device, dtype, top, shared):
+    """sigmoid scores, no renormalisation, weight on the expert's INPUT,
+    clamped activation, shared expert with its own limit and gate."""
+    width = 48
+    spec = moe(ff=20, limit=1.1, experts=6, top=top, shared=shared)
+    cfg = make_cfg([(delta(), spec)], width=width)
+    W = make_weights(cfg, seed=7)
+    h = rnd((17, width), 5, 1.5)
+    want = O.moe_ff(h, W, "l0.mlp.", spec)
+    ms = nx._mlp_spec(spec)
+    assert isinstance(ms, MlpSpec) and ms.weight_on_input
+    m = SparseMoE(width, ms, TD[dtype])
+    with torch.no_grad():
+        m.router.copy_(W["l0.mlp.router"])
+        for e in range(6):
+            m.experts_gate_up[e].copy_(torch.cat(
+                [W[f"l0.mlp.e{e}.gate"], W[f"l0.mlp.e{e}.up"]]))
+            m.experts_down[e].copy_(W[f"l0.mlp.e{e}.down"])
+        if shared:
+            m.shared.gate_up.copy_(torch.cat(
+                [W["l0.mlp.shared.gate"], W["l0.mlp.shared.up"]]))
+            m.shared.down.copy_(W["l0.mlp.shared.down"])
+            m.shared_gate.copy_(W["l0.mlp.shared.sg"])
+    m = m.to(device)
+    got = m(h.to(TD[dtype]).to(device))
+    # the clamp must bite for the test to mean anything
+    assert float(O.lin(W["l0.mlp.e0.gate"], h).max()) > 1.1
+    assert rel_err(got, want) < TOL[dtype]
+
+
+def test_weight_on_input_differs_from_weight_on_output():
+    """Guards the oracle itself: with a nonlinear expert, scaling the
+    input is not scaling the output."""
+    spec = moe(ff=20, limit=1.1, experts=3, top=1, shared=None)
+    cfg = make_cfg([(delta(), spec)], width=32)
+    W = make_weights(cfg, seed=8)
+    W["l0.mlp.router"] = (W["l0.mlp.router"].float() * 0.05).to(
+        torch.bfloat16)                       # scores near 1/2
+    h = rnd((5, 32), 6, 1.5)
+    a = O.moe_ff(h, W, "l0.mlp.", spec)
+    s = torch.sigmoid(O.lin(W["l0.mlp.router"], h))
+    b = torch.zeros_like(a)
+    for t in range(5):
+        e = int(s[t].argmax())
+        b[t] = s[t, e] * O.expert_ff(
+            h[t:t + 1], W[f"l0.mlp.e{e}.gate"], W[f"l0.mlp.e{e}.up"],
+            W[f"l0.mlp.e{e}.down"], 1.1)[0]
+    assert rel_err(b, a) > 0.05
+
+
+# ---------------------------------------------------------------------------
+# mixers: a tiny paged cache / slot harness
+# ---------------------------------------------------------------------------
+class Harness:
+    """Drives one mixer module over chosen portions of chosen sequences,
+    with scattered block tables and state slots, as the runner would."""
+
+    def __init__(self, mixer, device, dtype, n_seqs=3, max_len=400, bs=16,
+                 slots=4):
+        self.mixer, self.device, self.bs = mixer, device, bs
+        per = (max_len + bs - 1) // bs
+        g = torch.Generator().manual_seed(99)
+        nb = per * n_seqs + 5
+        perm = torch.randperm(nb, generator=g)
+        self.tables = perm[:per * n_seqs].view(n_seqs, per).to(torch.int32)
+        kind, a, b, c = mixer.cache_shape()
+        if kind == "kv":
+            # garbage in every page: stale keys must never be read
+            self.cache = (
+                torch.randn(nb, a, bs, b, generator=g).to(dtype).to(device),
+                torch.randn(nb, a, bs, c, generator=g).to(dtype).to(device))
+        else:
+            self.cache = torch.randn(slots, a, b, c, generator=g).to(device)
+
+    def run(self, parts, slot_of=None):
+        """parts: [(seq index, first position, projections [n, rows])];
+        returns the mixer's outputs, one tensor per part."""
+        bs, dev = self.bs, self.device
+        proj = torch.cat([p for _, _, p in parts]).to(dev)
+        pos, tseq, slots, rows = [], [], [], []
+        r0 = 0
+        for i, (s, p0, p) in enumerate(parts):
+            n = p.shape[0]
+            for t in range(n):
+                pp = p0 + t
+                pos.append(pp)
+                tseq.append(i)
+                slots.append(int(self.tables[s][pp // bs]) * bs + pp % bs)
+            rows.append([r0, n, p0, (slot_of or {}).get(s, s)])
+            r0 += n
+        meta = BatchMeta(
+            positions=torch.tensor(pos, dtype=torch.int32, device=dev),
+            slot_mapping=torch.tensor(slots, dtype=torch.long, device=dev),
+            num_prefill_tokens=0, prefill_token_seq=None,
+            prefill_token_pos=None, prefill_block_tables=None,
+            num_decode_seqs=0, decode_seq_lens=None,
+            decode_block_tables=None,
+            block_tables=torch.stack(
+                [self.tables[s] for s, _, _ in parts]).to(dev),
+            token_seq=torch.tensor(tseq, dtype=torch.int32, device=dev),
+            seq_rows=torch.tensor(rows, dtype=torch.int32, device=dev))
+        out = self.mixer.forward_from_proj(proj, meta, self.cache)
+        res, r0 = [], 0
+        for _, _, p in parts:
+            res.append(out[r0:r0 + p.shape[0]])
+            r0 += p.shape[0]
+        return res
+
+
+def build(kind_layer, width, W, dtype, device, eps=1e-5, rank=8):
+    cfg = make_cfg([(kind_layer, None)], width=width)
+    mcfg = nx.config_from_json(cfg, decay_ranks={0: rank})
+    mixer = build_mixer(width, mcfg.layer_specs[0].mixer, eps, TD[dtype])
+    with torch.no_grad():
+        if mixer.kind == "attention":
+            mixer.qkv.copy_(torch.cat(
+                [W["l0.mix.q"], W["l0.mix.k"], W["l0.mix.v"]]))
+            mixer.talk.copy_(W["l0.mix.talk"])
+        else:
+            mixer.in_proj.copy_(torch.cat(
+                [W["l0.mix." + n] for n in ("r", "k", "v", "g", "a", "w1")]))
+            mixer.w2.copy_(W["l0.mix.w2"])
+            mixer.w0.copy_(W["l0.mix.w0"])
+            mixer.a_bias.copy_(W["l0.mix.a.b"])
+            mixer.out_norm.copy_(W["l0.mix.norm"])
+        mixer.out_weight.copy_(W["l0.mix.o"])
+    return mixer.to(device)
+
+
+def project(mixer, h, dtype, device):
+    w = torch.cat([p.data for p in mixer.in_params()])
+    return torch.nn.functional.linear(h.to(TD[dtype]).to(device), w)
+
+
+def finish(mixer, outs):
+    return torch.nn.functional.linear(torch.cat(outs), mixer.out_weight)
+
+
+PORTIONS = [[None], [1] * 12 + [None], [2, 3, 2, 17, 5, None],
+            [16, 16, 1, 1, None], [31, 2, None]]
+
+
+def split(n, sizes):
+    cuts, at = [], 0
+    for s in sizes:
+        s = n - at if s is None else min(s, n - at)
+        if s > 0:
+            cuts.append((at, at + s))
+            at += s
+    return cuts
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim", [(3, 16), (1, 24), (2, 40)])
+def test_general_delta_mixer(device, dtype, heads, dim):
+    width, T = 56, 75
+    layer = delta(heads, dim)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=11)
+    h = rnd((T, width), 12, 1.2)
+    want, _ = O.general_delta(h, W, "l0.mix.", layer["mixer"], 1e-5)
+    mixer = build(layer, width, W, dtype, device)
+    proj = project(mixer, h, dtype, device)
+    for sizes in PORTIONS:
+        hz = Harness(mixer, device, TD[dtype])
+        outs = []
+        for a, b in split(T, sizes):
+            outs += hz.run([(1, a, proj[a:b])])
+        assert rel_err(finish(mixer, outs), want) < TOL[dtype], sizes
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_general_delta_state_survives_long_gaps(device):
+    """Decay pinned near 1 and removal near 0: what the first tokens wrote
+    must still be read hundreds of tokens later, across many portions; a
+    dropped or re-zeroed state would change the read-out completely."""
+    width, T = 32, 330
+    layer = delta(2, 16)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=13)
+    W["l0.mix.w0"] = torch.full_like(W["l0.mix.w0"], -9.0)   # decay ~ 1
+    W["l0.mix.w2"] = torch.zeros_like(W["l0.mix.w2"])
+    W["l0.mix.a.b"] = torch.full_like(W["l0.mix.a.b"], -9.0)  # no removal
+    W["l0.mix.a"] = torch.zeros_like(W["l0.mix.a"])
+    h = rnd((T, width), 14, 0.2)
+    h[:3] = rnd((3, width), 15, 6.0)        # loud first tokens
+    want, _ = O.general_delta(h, W, "l0.mix.", layer["mixer"], 1e-5)
+    quiet = h.clone()
+    quiet[:3] = 0
+    other, _ = O.general_delta(quiet, W, "l0.mix.", layer["mixer"], 1e-5)
+    assert rel_err(other[300:], want[300:]) > 0.5   # the test has teeth
+    mixer = build(layer, width, W, "float32", device)
+    proj = project(mixer, h, "float32", device)
+    hz = Harness(mixer, device, torch.float32)
+    outs = []
+    for a, b in split(T, [3, 64, 2, 1, 1, 100, 7, 1, 1, 1, None]):
+        outs += hz.run([(0, a, proj[a:b])])
+    assert rel_err(finish(mixer, outs), want) < TOL["float32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_general_delta_batch_and_slot_reuse(device):
+    """Unequal sequences in one launch equal each alone; a slot handed to
+    a new sequence starts from zero although it holds an old state."""
+    width = 48
+    layer = delta(3, 16)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=16)
+    hs = [rnd((n, width), 20 + i, 1.2) for i, n in enumerate((41, 9, 1))]
+    wants = [O.general_delta(h, W, "l0.mix.", layer["mixer"], 1e-5)[0]
+             for h in hs]
+    mixer = build(layer, width, W, "float32", device)
+    pj = [project(mixer, h, "float32", device) for h in hs]
+    hz = Harness(mixer, device, torch.float32)
+    slot_of = {0: 2, 1: 0, 2: 3}
+    o1 = hz.run([(0, 0, pj[0][:30]), (1, 0, pj[1][:8]), (2, 0, pj[2])],
+                slot_of)
+    o2 = hz.run([(1, 8, pj[1][8:]), (0, 30, pj[0][30:])], slot_of)
+    assert rel_err(finish(mixer, [o1[0], o2[1]]), wants[0]) < 2e-4
+    assert rel_err(finish(mixer, [o1[1], o2[0]]), wants[1]) < 2e-4
+    assert rel_err(finish(mixer, [o1[2]]), wants[2]) < 2e-4
+    # sequence 2's slot now goes to a fresh copy of sequence 1
+    o3 = hz.run([(1, 0, pj[1])], {1: 3})
+    assert rel_err(finish(mixer, o3), wants[1]) < 2e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layer", [
+    attn(6, 2, 16, 24, 20, 0.3), attn(3, 3, 24, 8, 33, 0.2),
+    attn(4, 1, 8, 16, 16, 0.4), attn(2, 2, 32, 32, 500, 0.15)])
+def test_attention_mixer(device, dtype, layer):
+    width, T = 56, 75
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=31)
+    h = rnd((T, width), 32, 1.2)
+    want = O.attention(h, W, "l0.mix.", layer["mixer"])
+    mixer = build(layer, width, W, dtype, device)
+    proj = project(mixer, h, dtype, device)
+    for sizes in PORTIONS:
+        hz = Harness(mixer, device, TD[dtype])
+        outs = []
+        for a, b in split(T, sizes):
+            outs += hz.run([(2, a, proj[a:b])])
+        assert rel_err(finish(mixer, outs), want) < TOL[dtype], sizes
+
+
+def needle_setup(size, T, needle, width=40):
+    """Tied query/key weights and inputs close to the needle's make the
+    needle's score tower over every other key's."""
+    layer = attn(2, 2, 16, 16, size, 0.25)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=41)
+    W["l0.mix.k"] = W["l0.mix.q"].clone()
+    W["l0.mix.talk"] = torch.eye(2).to(torch.bfloat16)
+    base = rnd((1, width), 42, 1.0)
+    h = (base * 0.05 + rnd((T, width), 43, 0.05)).to(torch.bfloat16)
+    h[needle] = base[0] * 3.0
+    for i in range(needle + 1, T):
+        h[i] = (h[i].float() + base[0].float() * 1.0).to(torch.bfloat16)
+    return layer, W, h
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("size,needle,probe,seen", [
+    (48, 47, [48, 49], False),   # needle just outside the probes' chunk
+    (48, 48, [49, 95], True),    # needle is the chunk's first key
+    (48, 48, [96, 97], False),   # ... and gone again one chunk later
+    (48, 95, [95], True),        # the chunk's last position sees itself
+    (512, 3, [400, 470], True),  # far back, many pages away, still seen
+])
+def test_attention_chunk_edges_with_needle(device, size, needle, probe,
+                                           seen):
+    T = max(probe) + 1
+    layer, W, h = needle_setup(size, T, needle)
+    want = O.attention(h, W, "l0.mix.", layer["mixer"])
+    # where the needle is seen it decides the output, elsewhere it must
+    # not touch it: a visibility edge off by one key would show
+    dull = h.clone()
+    dull[needle] = h[needle - 1] if needle else h[needle + 1]
+    shift = rel_err(O.attention(dull, W, "l0.mix.", layer["mixer"])[probe],
+                    want[probe])
+    if seen:
+        assert shift > 0.2
+    elif needle not in probe:
+        assert shift < 1e-9
+    mixer = build(layer, 40, W, "float32", device)
+    proj = project(mixer, h, "float32", device)
+    first = min(probe)
+    for sizes in ([None], [first, 1, None], [first - 1, 2, None],
+                  [needle, 1] + [1] * (T - needle)):
+        hz = Harness(mixer, device, torch.float32, max_len=T + 16)
+        outs = []
+        for a, b in split(T, sizes):
+            outs += hz.run([(0, a, proj[a:b])])
+        got = finish(mixer, outs)
+        assert rel_err(got[probe], want[probe]) < 2e-4, sizes
+        assert rel_err(got, want) < 2e-4, sizes
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_attention_sink_takes_weight(device):
+    """With every score far below 0 the sink holds nearly all the weight
+    and the output is nearly 0 instead of a mean of values; the first key
+    of a chunk alone gets e^s / (1 + e^s)."""
+    width, T = 32, 40
+    layer = attn(2, 1, 16, 16, 20, 0.5)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=51)
+    W["l0.mix.k"] = (-W["l0.mix.q"][:16].float()).to(torch.bfloat16)
+    W["l0.mix.q"][16:] = W["l0.mix.q"][:16]
+    W["l0.mix.talk"] = torch.eye(2).to(torch.bfloat16)
+    base = rnd((1, width), 52, 1.0)
+    h = (base * 2.0 + rnd((T, width), 53, 0.05)).to(torch.bfloat16)
+    want = O.attention(h, W, "l0.mix.", layer["mixer"])
+    v = O.lin(W["l0.mix.v"], h)
+    assert float(want.abs().max()) < 0.05 * float(
+        O.lin(W["l0.mix.o"], torch.cat([v, v], -1)).abs().max())
+    mixer = build(layer, width, W, "float32", device)
+    proj = project(mixer, h, "float32", device)
+    hz = Harness(mixer, device, torch.float32)
+    outs = []
+    for a, b in split(T, [19, 1, 1, 2, None]):
+        outs += hz.run([(0, a, proj[a:b])])
+    got = finish(mixer, outs)
+    assert float((got.double().cpu() - want).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_attention_head_mixing_matters(device):
+    """A far-from-identity mixing matrix (one head's scores are mostly
+    another's) against the oracle; unmixed scores would be far off."""
+    width, T = 40, 30
+    layer = attn(4, 2, 16, 8, 12, 0.3)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=61)
+    W["l0.mix.talk"] = torch.tensor(
+        [[0.1, 1.2, 0.0, -0.5], [0.9, 0.0, 0.6, 0.0],
+         [0.0, -0.7, 0.2, 1.0], [0.5, 0.5, 0.5, 0.5]]).to(torch.bfloat16)
+    h = rnd((T, width), 62, 1.5)
+    want = O.attention(h, W, "l0.mix.", layer["mixer"])
+    plain = dict(W)
+    plain["l0.mix.talk"] = torch.eye(4).to(torch.bfloat16)
+    assert rel_err(O.attention(h, plain, "l0.mix.", layer["mixer"]),
+                   want) > 0.2
+    mixer = build(layer, width, W, "float32", device)
+    proj = project(mixer, h, "float32", device)
+    hz = Harness(mixer, device, torch.float32)
+    got = finish(mixer, hz.run([(1, 0, proj[:11])])
+                 + hz.run([(1, 11, proj[11:])]))
+    assert rel_err(got, want) < 2e-4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_attention_batch_of_unequal_requests(device):
+    width = 48
+    layer = attn(6, 3, 16, 24, 20, 0.3)
+    W = make_weights(make_cfg([(layer, None)], width=width), seed=71)
+    hs = [rnd((n, width), 72 + i, 1.2) for i, n in enumerate((45, 21, 1))]
+    wants = [O.attention(h, W, "l0.mix.", layer["mixer"]) for h in hs]
+    mixer = build(layer, width, W, "float32", device)
+    pj = [project(mixer, h, "float32", device) for h in hs]
+    hz = Harness(mixer, device, torch.float32)
+    o1 = hz.run([(0, 0, pj[0][:19]), (1, 0, pj[1][:20]), (2, 0, pj[2])])
+    o2 = hz.run([(1, 20, pj[1][20:]), (0, 19, pj[0][19:21])])
+    o3 = hz.run([(0, 21, pj[0][21:])])
+    assert rel_err(finish(mixer, [o1[0], o2[1], o3[0]]), wants[0]) < 2e-4
+    assert rel_err(finish(mixer, [o1[1], o2[0]]), wants[1]) < 2e-4
+    assert rel_err(finish(mixer, [o1[2]]), wants[2]) < 2e-4

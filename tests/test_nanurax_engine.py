@@ -1,0 +1,269 @@
+"""Nanurax through the engine: checkpoint folder -> registry -> runner ->
+scheduler / block manager / state slots, against the float64 oracle. Every
+test builds its own small configuration and random weights. CPU runs the
+reference ops; gpu-marked variants run the HIP kernels."""
+
+import json
+
+import pytest
+import torch
+
+import oracle_nanurax as O
+from nanurax_util import (TOL, attn, delta, dense, make_cfg, make_engine,
+                          make_weights, moe, rel_err, save_checkpoint)
+from nanurax_util import close
+from production_stack_amd.engine.block_manager import BlockManager
+from production_stack_amd.engine.models import registry
+from production_stack_amd.engine.sampling import SamplingParams
+from production_stack_amd.engine.sequence import Sequence
+
+pytestmark = pytest.mark.filterwarnings("ignore::UserWarning")
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DTYPES = ["float32", "bfloat16"]
+
+# a stack that differs from any single-valued choice: head counts and dims
+# vary by layer, group sizes 3 and 1, value width != key width, two and
+# three experts per token, a layer without feed-forward, routed layers with
+# and without a shared expert, attention first and last
+STACK = [
+    (attn(6, 2, 16, 24, 20, 0.3), dense(72)),
+    (delta(3, 16), moe(24, 1.75, 5, 2, (40, 1.25))),
+    (delta(2, 24), None),
+    (attn(3, 3, 8, 8, 33, 0.45), moe(16, 0.9, 4, 3, None)),
+    (delta(1, 40), dense(56)),
+]
+
+
+@pytest.fixture(scope="module")
+def ckpt(tmp_path_factory):
+    cfg = make_cfg(STACK, width=64, vocab=97)
+    W = make_weights(cfg, seed=5, rank=6)
+    path = save_checkpoint(tmp_path_factory.mktemp("nx") / "m", cfg, W)
+    return path, cfg, W
+
+
+def tokens(n, seed, vocab=97):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def replay(eng, rid, toks, sizes, want_all=True):
+    """Feed toks in portions of the given sizes (None = the rest); returns
+    logits at every position."""
+    out, at = [], 0
+    for s in sizes:
+        s = len(toks) - at if s is None else min(s, len(toks) - at)
+        if s <= 0:
+            continue
+        last = at + s == len(toks)
+        out.append(eng.replay_step(
+            [(rid, toks[at:at + s], list(range(s)))],
+            end=[rid] if last else []))
+        at += s
+    assert at == len(toks)
+    return torch.cat(out)
+
+
+# ---------------------------------------------------------------------------
+def test_registry_reads_checkpoint_folder(ckpt):
+    path, cfg, W = ckpt
+    mc = registry.config_from_dir(path)
+    assert mc.family == "nanurax" and mc.vocab_size == 97
+    assert mc.hidden_size == 64 and len(mc.layer_specs) == len(STACK)
+    s0, s1, s2, s3 = mc.layer_specs[:4]
+    assert (s0.mixer.kind, s0.mixer.heads, s0.mixer.kv_heads,
+            s0.mixer.vdim, s0.mixer.chunk) == ("attention", 6, 2, 24, 20)
+    assert s0.mixer.sink and s0.mixer.talking_heads and not s0.mixer.rope
+    assert s1.mixer.decay_rank == 6          # read off the tensor's shape
+    assert (s1.mlp.experts, s1.mlp.top, s1.mlp.shared_ff,
+            s1.mlp.shared_limit) == (5, 2, 40, 1.25)
+    assert s1.mlp.score == "sigmoid" and not s1.mlp.renormalize
+    assert s2.mlp is None and s3.mlp.shared_ff == 0
+    assert mc.has_recurrent_state
+    with open(path + "/config.json") as f:
+        bad = json.load(f)
+    bad["architecture"] = "Nope"
+    import os
+    os.makedirs(path + "_bad", exist_ok=True)
+    with open(path + "_bad/config.json", "w") as f:
+        json.dump(bad, f)
+    with pytest.raises(ValueError):
+        registry.config_from_dir(path + "_bad")
+
+
+def test_state_slot_pool():
+    bm = BlockManager(32, 16, enable_prefix_caching=True, num_state_slots=2)
+    assert not bm.enable_prefix_caching   # recurrent state: no prefix reuse
+    sp = SamplingParams(max_tokens=1)
+    a, b, c = (Sequence(n, [1] * 20, sp) for n in "abc")
+    bm.allocate_prompt(a)
+    bm.allocate_prompt(b)
+    assert {a.state_slot, b.state_slot} == {0, 1}
+    assert not bm.can_allocate_prompt(c)  # blocks are free, slots are not
+    with pytest.raises(RuntimeError):
+        bm.allocate_prompt(c)
+    assert bm.num_free == 32 - 4          # the failed admission leaked none
+    freed = a.state_slot
+    bm.free_seq(a)
+    assert a.state_slot is None and bm.can_allocate_prompt(c)
+    bm.allocate_prompt(c)
+    assert c.state_slot == freed
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole_prompt_and_every_layer(ckpt, device, dtype):
+    path, cfg, W = ckpt
+    toks = tokens(70, 1)
+    want, layers = O.forward(cfg, W, toks, return_layers=True)
+    eng = make_engine(path, dtype, device)
+    seen = {}
+    eng.runner.model.residual_hook = lambda i, x: seen.__setitem__(
+        i, x.detach().clone())
+    got = replay(eng, "a", toks, [None])
+    assert close(got, want, dtype)
+    assert sorted(seen) == list(range(len(STACK)))
+    for i in range(len(STACK)):
+        assert seen[i].dtype == torch.float32     # fp32 residual stream
+        assert close(seen[i], layers[i], dtype), i
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens_and_single_token_prompt(ckpt, device, dtype):
+    path, cfg, W = ckpt
+    eng = make_engine(path, dtype, device)
+    for n in (1, 2, 3):
+        toks = tokens(n, 10 + n)
+        want = O.forward(cfg, W, toks)
+        assert close(replay(eng, f"p{n}", toks, [None]), want, dtype)
+        assert close(replay(eng, f"q{n}", toks, [1] * n), want, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [
+    [1] * 90, [2] * 45, [3, 2, 17, 2, 31, 2, None], [19, 1, 1, 1, None],
+    [20, 20, 13, None], [33, 33, None], [16, 16, 16, 16, 16, None]])
+def test_portions_match_whole_prompt(ckpt, device, dtype, sizes):
+    """Prefill against token-by-token decoding, and portions of several
+    sizes down to two tokens, cut inside pages and chunks and exactly on
+    their edges (chunks of 20 and 33 positions, pages of 16)."""
+    path, cfg, W = ckpt
+    toks = tokens(90, 2)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, dtype, device)
+    assert close(replay(eng, "a", toks, sizes), want, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decode_past_many_chunks(ckpt, device):
+    path, cfg, W = ckpt
+    toks = tokens(260, 3)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, "float32", device)
+    got = replay(eng, "a", toks, [37] + [1] * 223)
+    assert rel_err(got, want) < TOL["float32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mixed_batches_reuse_pages_and_slots(ckpt, device, dtype):
+    """Up to three live requests of unequal length per step, portions
+    beside single tokens; the pool (3 slots, 12 pages) is smaller than the
+    sum of all requests, so pages and slots pass from finished requests to
+    new ones. Every request must equal itself alone."""
+    path, cfg, W = ckpt
+    lens = {"a": 61, "b": 5, "c": 40, "d": 1, "e": 47, "f": 22}
+    toks = {k: tokens(n, 30 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: O.forward(cfg, W, v) for k, v in toks.items()}
+    eng = make_engine(path, dtype, device, blocks=12, max_seqs=3)
+    plan = [
+        [("a", 17), ("b", 2), ("c", 3)],
+        [("a", 1), ("b", 3), ("c", 16)],          # b ends
+        [("a", 2), ("d", 1), ("c", 1)],           # d: one-token request
+        [("c", 20), ("e", 31)],                   # a sits out; c ends
+        [("a", 41), ("e", 1), ("f", 2)],          # a ends
+        [("e", 15), ("f", 20)],                   # both end
+    ]
+    at = {k: 0 for k in toks}
+    got = {k: [] for k in toks}
+    for step in plan:
+        entries, end = [], []
+        for rid, n in step:
+            lo = at[rid]
+            entries.append((rid, toks[rid][lo:lo + n], list(range(n))))
+            at[rid] += n
+            if at[rid] == lens[rid]:
+                end.append(rid)
+        out = eng.replay_step(entries, end=end)
+        r0 = 0
+        for rid, n in step:
+            got[rid].append(out[r0:r0 + n])
+            r0 += n
+    assert at == lens
+    bm = eng.block_manager
+    assert bm.num_free == 12 and len(bm.free_slots) == 3   # all given back
+    for k in toks:
+        assert close(torch.cat(got[k]), want[k], dtype), k
+
+
+def test_replay_refuses_a_plan_that_does_not_fit(ckpt):
+    path, cfg, W = ckpt
+    eng = make_engine(path, "float32", "cpu", blocks=4, max_seqs=2)
+    eng.replay_step([("a", tokens(10, 1), []), ("b", tokens(10, 2), [])])
+    with pytest.raises(RuntimeError):
+        eng.replay_step([("c", tokens(3, 3), [])])       # no slot left
+    with pytest.raises(RuntimeError):
+        eng.replay_step([("a", tokens(60, 4), [])])      # no pages left
+
+
+def oracle_greedy(cfg, W, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(O.forward(cfg, W, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("budget,blocks", [(1 << 20, 64), (7, 64), (24, 9)])
+def test_greedy_generation_through_the_scheduler(ckpt, device, budget,
+                                                 blocks):
+    """LLMEngine.generate: the scheduler's own chunking (token budgets of
+    7 and 24 cut the prompts into portions), continuous batching of three
+    unequal requests, and with 9 pages preemption with recomputation, must
+    all give the oracle's greedy continuation."""
+    path, cfg, W = ckpt
+    prompts = [tokens(45, 50), tokens(3, 51), tokens(28, 52)]
+    n_new = 12
+    want = [oracle_greedy(cfg, W, p, n_new) for p in prompts]
+    eng = make_engine(path, "float32", device, blocks=blocks, max_seqs=3,
+                      budget=budget)
+    out = eng.generate(prompts, SamplingParams(
+        max_tokens=n_new, temperature=0.0, ignore_eos=True))
+    for i in range(3):
+        assert out[f"offline-{i}"] == want[i], i
+    assert eng.block_manager.num_free == blocks
+    assert len(eng.block_manager.free_slots) == 3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_other_layer_orders_and_sizes(tmp_path, device):
+    """A second stack: recurrent layers only at the ends, one expert per
+    token beside many, a chunk of one position (a key sees only itself),
+    width that is no multiple of 64."""
+    stack = [
+        (delta(4, 8), moe(8, 2.5, 7, 1, (8, 0.5))),
+        (attn(2, 1, 24, 16, 1, 0.2), None),
+        (attn(8, 4, 8, 16, 64, 0.35), dense(40)),
+        (delta(2, 32), dense(24)),
+    ]
+    cfg = make_cfg(stack, width=72, vocab=53, eps=3e-4, scale=2.25)
+    W = make_weights(cfg, seed=9, rank=3)
+    path = save_checkpoint(tmp_path / "m2", cfg, W)
+    toks = tokens(80, 60, vocab=53)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, "float32", device)
+    assert rel_err(replay(eng, "a", toks, [None]), want) < 2e-4
+    assert rel_err(replay(eng, "b", toks, [5, 2, 60, 1, None]), want) < 2e-4
