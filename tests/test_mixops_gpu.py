@@ -106,7 +106,7 @@ def test_kv_append_distinct_widths(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,DV,chunk,window,sink,talk", [
-    (4, 2, 48, 48, 24, 0, True, True),
+    (4, 2, 40, 40, 24, 0, True, True),
     (6, 3, 40, 24, 40, 0, True, True),
     (3, 1, 32, 64, 0, 0, False, False),
     (4, 4, 16, 16, 0, 20, True, False),
@@ -145,7 +145,7 @@ def test_talk_attention(dtype, H, G, D, DV, chunk, window, sink, talk):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D", [(2, 48), (3, 16), (1, 72), (2, 128),
+@pytest.mark.parametrize("H,D", [(2, 56), (3, 16), (1, 72), (2, 128),
                                  (1, 160)])
 def test_delta_rule(dtype, H, D):
     g = torch.Generator().manual_seed(5)
