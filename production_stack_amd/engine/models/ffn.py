@@ -32,11 +32,14 @@ def route(x: torch.Tensor, router_w: torch.Tensor, top: int,
     logits = F.linear(x.float(), router_w.float())
     if score == "softmax":
         probs = torch.softmax(logits, dim=-1)
+        weights, sel = torch.topk(probs, top, dim=-1)
     elif score == "sigmoid":
-        probs = torch.sigmoid(logits)
+        # rank by the logits: the sigmoid is monotonic but saturates to
+        # exactly 1.0 in fp32, which would tie large scores
+        _, sel = torch.topk(logits, top, dim=-1)
+        weights = torch.sigmoid(logits.gather(-1, sel))
     else:
         raise ValueError(f"unknown router score {score!r}")
-    weights, sel = torch.topk(probs, top, dim=-1)
     if renormalize:
         weights = weights / weights.sum(dim=-1, keepdim=True)
     return weights, sel

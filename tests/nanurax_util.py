@@ -94,7 +94,7 @@ def make_weights(cfg, seed=0, rank=8):
                 lin(f"{p}mlp.e{e}.gate", ff, width, 3.0)
                 lin(f"{p}mlp.e{e}.up", ff, width, 3.0)
                 lin(f"{p}mlp.e{e}.down", width, ff)
-            lin(p + "mlp.router", f["router"]["experts"], width, 8.0)
+            lin(p + "mlp.router", f["router"]["experts"], width, 4.0)
             if f.get("shared"):
                 sf = f["shared"]["ff"]
                 lin(p + "mlp.shared.gate", sf, width, 3.0)
