@@ -377,6 +377,67 @@ ARCHITECTURES = {
 }
 
 
+def _nanurax_stack(
+    name: str, width: int, vocab: int, n_layers: int, *, delta_heads: int,
+    delta_dim: int, decay_rank: int, attn_heads: int, attn_kv: int,
+    attn_dim: int, chunk: int, ff: int, experts: int, top: int,
+    expert_ff: int, shared_ff: int, limit: float = 7.0,
+) -> ModelConfig:
+    """A Nanurax stack in the repeating order delta+dense, delta+routed,
+    attention+dense, delta+routed (three recurrent layers per attention
+    layer, every other feed-forward routed)."""
+    pattern = [("general_delta", "dense"), ("general_delta", "moe"),
+               ("attention", "dense"), ("general_delta", "moe")]
+    specs = []
+    for i in range(n_layers):
+        mk, fk = pattern[i % len(pattern)]
+        if mk == "attention":
+            mixer = MixerSpec(
+                kind="attention", heads=attn_heads, dim=attn_dim,
+                kv_heads=attn_kv, vdim=attn_dim,
+                scale=attn_dim ** -0.5, chunk=chunk, sink=True,
+                talking_heads=True, rope=False)
+        else:
+            mixer = MixerSpec(kind="general_delta", heads=delta_heads,
+                              dim=delta_dim, rope=False,
+                              decay_rank=decay_rank)
+        if fk == "dense":
+            mlp = MlpSpec(kind="dense", ff=ff, act="gelu_tanh")
+        else:
+            mlp = MlpSpec(
+                kind="moe", ff=expert_ff, act="clamped_swish", limit=limit,
+                experts=experts, top=top, score="sigmoid",
+                renormalize=False, weight_on_input=True,
+                shared_ff=shared_ff, shared_limit=limit)
+        specs.append(LayerSpec(mixer=mixer, mlp=mlp, parallel=True))
+    return ModelConfig(
+        name=name, family="nanurax", hidden_size=width,
+        num_layers=n_layers, num_q_heads=attn_heads, num_kv_heads=attn_kv,
+        head_dim=attn_dim, intermediate_size=ff, vocab_size=vocab,
+        max_position=1 << 20, layer_specs=specs,
+        embedding_scale=float(width) ** 0.5, bos_token_id=0,
+        eos_token_id=-1)
+
+
+ARCHITECTURES.update({
+    # CPU-runnable test config
+    "tiny-nanurax": _nanurax_stack(
+        "tiny-nanurax", 64, 512, 4, delta_heads=2, delta_dim=16,
+        decay_rank=8, attn_heads=4, attn_kv=2, attn_dim=16, chunk=32,
+        ff=128, experts=4, top=2, expert_ff=32, shared_ff=64),
+    # llama-3.2-1b-sized stack (same width, depth, dense ff and vocab)
+    "nanurax-1b": _nanurax_stack(
+        "nanurax-1b", 2048, 128256, 16, delta_heads=32, delta_dim=64,
+        decay_rank=64, attn_heads=32, attn_kv=8, attn_dim=64, chunk=1024,
+        ff=8192, experts=8, top=2, expert_ff=2048, shared_ff=2048),
+    # llama-3-8b-sized layers (width 4096, head dim 128, ff 14336)
+    "nanurax-8b": _nanurax_stack(
+        "nanurax-8b", 4096, 128256, 32, delta_heads=32, delta_dim=128,
+        decay_rank=64, attn_heads=32, attn_kv=8, attn_dim=128, chunk=2048,
+        ff=14336, experts=8, top=2, expert_ff=3584, shared_ff=3584),
+})
+
+
 @dataclass
 class CacheConfig:
     block_size: int = 16
