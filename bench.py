@@ -110,8 +110,122 @@ class User:
         self.history.extend(answer_tokens)
 
 
+# --compare-family: prefill / decode throughput of a model family beside the
+# closest Llama config at equal width, depth, dense-ff width and vocabulary
+COMPARE_PAIRS = {
+    "nanurax": [("nanurax-1b", "llama-3.2-1b"), ("nanurax-8b", "llama-3-8b")],
+}
+
+
+def _truncated(name: str, layers: int) -> str:
+    """Register `name` cut to its first `layers` layers; returns the new
+    architecture name (layer shapes are what is compared, so a few layers
+    of each are enough and keep the run short)."""
+    import dataclasses
+
+    from production_stack_amd.engine.config import ARCHITECTURES
+
+    cfg = ARCHITECTURES[name]
+    if layers <= 0 or layers >= cfg.num_layers:
+        return name
+    new = f"{name}-L{layers}"
+    kw = {"name": new, "num_layers": layers}
+    if cfg.layer_specs:
+        kw["layer_specs"] = cfg.layer_specs[:layers]
+    ARCHITECTURES[new] = dataclasses.replace(cfg, **kw)
+    return new
+
+
+def _compare_one(model: str, args, use_cuda: bool) -> dict:
+    L, P = args.compare_prompt_len, args.compare_prompts
+    B, ctx, new = args.compare_batch, args.compare_context, 32
+    cfg = EngineConfig(
+        model=model,
+        max_model_len=max(L, ctx + new) + 64,
+        seed=1234,
+        cache=CacheConfig(
+            block_size=16, enable_prefix_caching=False,
+            num_gpu_blocks=(max(P * L, B * (ctx + new)) // 16 + 4 * B + 64),
+        ),
+        scheduler=SchedulerConfig(max_num_seqs=max(B, P),
+                                  max_num_batched_tokens=8192,
+                                  max_prefill_chunk=8192),
+    )
+    engine = LLMEngine(cfg, device=None if use_cuda else "cpu")
+    rng = np.random.default_rng(7)
+    hi = min(VOCAB_HIGH, engine.model_cfg.vocab_size - 1)
+
+    def sync():
+        if use_cuda:
+            torch.cuda.synchronize()
+
+    def prompts(n, length):
+        return [rng.integers(VOCAB_LOW, hi, size=length).tolist()
+                for _ in range(n)]
+
+    one = SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True)
+    engine.generate(prompts(1, min(L, 512)), one)       # warm-up
+    sync()
+    t0 = time.perf_counter()
+    engine.generate(prompts(P, L), one)
+    sync()
+    prefill = P * L / (time.perf_counter() - t0)
+
+    many = SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True)
+    for i, pr in enumerate(prompts(B, ctx)):
+        engine.add_request(f"d{i}", pr, many)
+    live = {f"d{i}" for i in range(B)}
+    started: set = set()
+    while len(started) < B:                              # prefill phase
+        for out in engine.step():
+            if out.new_token_ids:
+                started.add(out.request_id)
+    sync()
+    t0 = time.perf_counter()
+    toks = 0
+    while engine.has_unfinished():
+        for out in engine.step():
+            toks += len(out.new_token_ids)
+    sync()
+    decode = toks / (time.perf_counter() - t0)
+    del engine
+    if use_cuda:
+        torch.cuda.empty_cache()
+    return {"model": model, "prefill_tokens_per_sec": round(prefill, 1),
+            "decode_tokens_per_sec": round(decode, 1),
+            "prefill": f"{P}x{L}", "decode": f"batch {B} @ ctx {ctx}"}
+
+
+def run_family_compare(args) -> None:
+    use_cuda = torch.cuda.is_available() and args.device != "cpu"
+    pairs = COMPARE_PAIRS[args.compare_family]
+    if args.compare_models:
+        pairs = [tuple(p.split(":")) for p in args.compare_models.split(",")]
+    rows = []
+    for new, base in pairs:
+        for name in (new, base):
+            model = _truncated(name, args.compare_layers)
+            r = _compare_one(model, args, use_cuda)
+            rows.append(r)
+            print(json.dumps(r), flush=True)
+    print(json.dumps({"metric": "family_compare", "dtype": "bf16",
+                      "data": "synthetic", "rows": rows}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--compare-family", default=None,
+                    choices=sorted(COMPARE_PAIRS),
+                    help="instead of the serving benchmark, measure prefill "
+                         "and decode throughput of this family beside the "
+                         "closest Llama config at equal size")
+    ap.add_argument("--compare-models", default=None,
+                    help="new:base[,new:base] architecture names")
+    ap.add_argument("--compare-layers", type=int, default=8)
+    ap.add_argument("--compare-prompt-len", type=int, default=4096)
+    ap.add_argument("--compare-prompts", type=int, default=4)
+    ap.add_argument("--compare-batch", type=int, default=64)
+    ap.add_argument("--compare-context", type=int, default=1024)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=48)
@@ -132,6 +246,9 @@ def main() -> None:
                     help="restore the split graph+eager mixed-step path "
                          "(unified reads weights once per step; default)")
     args = ap.parse_args()
+    if args.compare_family:
+        run_family_compare(args)
+        return
 
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

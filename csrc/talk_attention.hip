@@ -15,6 +15,18 @@
 
 #define TA_KT 32
 
+// Dynamic LDS a kernel may ask for: gfx950 has 160 KB per CU, but a launch
+// above 64 KB needs the limit raised per kernel first. Falls back to 64 KB
+// when the runtime refuses.
+static size_t ta_lds_budget(const void* fn) {
+  const int want = 160 * 1024;
+  if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          want) == hipSuccess)
+    return (size_t)want;
+  (void)hipGetLastError();
+  return 64 * 1024;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void talk_attn_kernel(
     T* __restrict__ out, int ldout, const T* __restrict__ q, int ldq,
@@ -116,6 +128,394 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
     MxElem<T>::st(out + (size_t)t * ldout + it, sacc[it] / sl[it / DV]);
 }
 
+// ---------------------------------------------------------------------------
+// Tiled variant: one thread per (head, query) pair.
+//
+// A workgroup takes QT = 256 / H consecutive batch rows with all H heads;
+// thread (h, i) keeps its query vector and its output accumulator in
+// registers (DP floats each, head widths padded up to DP). Rows of the
+// group that continue one sequence at consecutive positions form a run; a
+// run shares every key/value tile, staged once into LDS as fp32 and read by
+// the threads as wave-wide broadcasts (lanes of a wave hold few distinct
+// heads). Per tile: raw scores -> LDS, head mix from LDS, one online-softmax
+// rescale, P.V from the LDS value rows. Single decode tokens are runs of
+// one row.
+template <typename T, int DP>
+__global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
+    T* __restrict__ out, int ldout, const T* __restrict__ q, int ldq,
+    const T* __restrict__ kc, const T* __restrict__ vc,
+    const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ token_seq, const int* __restrict__ token_pos,
+    const float* __restrict__ talk, int T_total, int H, int G, int D, int DV,
+    int BS, float scale, int chunk, int window, int sink, int QT, int KT) {
+  extern __shared__ float lds[];
+  const int NP = H * QT;
+  float* sK = lds;                   // [KT][G][DP]
+  float* sV = sK + KT * G * DP;      // [KT][G][DP]
+  float* sS = sV + KT * G * DP;      // [KT][NP] raw scores
+  float* sM = sS + KT * NP;          // [KT][NP] mixed scores
+  float* sT = sM + KT * NP;          // [H*H]
+  int* s_seq = (int*)(sT + H * H);   // [QT]
+  int* s_pos = s_seq + QT;           // [QT]
+
+  const int tid = threadIdx.x;
+  const int row0 = blockIdx.x * QT;
+  const int nrows = min(QT, T_total - row0);
+  const int h = tid / QT, i = tid % QT;
+  const bool valid = tid < NP && i < nrows;
+  const int rep = H / G;
+  const int gk = valid ? h / rep : 0;
+
+  for (int c = tid; c < nrows; c += blockDim.x) {
+    s_seq[c] = token_seq[row0 + c];
+    s_pos[c] = token_pos[row0 + c];
+  }
+  if (talk != nullptr)
+    for (int c = tid; c < H * H; c += blockDim.x) sT[c] = talk[c];
+
+  float qv[DP], acc[DP];
+#pragma unroll
+  for (int d = 0; d < DP; ++d) {
+    qv[d] = (valid && d < D)
+                ? MxElem<T>::ld(q + (size_t)(row0 + i) * ldq + h * D + d)
+                : 0.f;
+    acc[d] = 0.f;
+  }
+  float m = sink ? 0.f : PS_NEG_INF;
+  float l = sink ? 1.f : 0.f;
+  __syncthreads();
+  const int my_pos = valid ? s_pos[i] : 0;
+  int my_lo = 0;
+  if (chunk > 0) my_lo = (my_pos / chunk) * chunk;
+  if (window > 0) my_lo = max(my_lo, my_pos - window + 1);
+
+  int rs = 0;
+  while (rs < nrows) {
+    int re = rs + 1;
+    while (re < nrows && s_seq[re] == s_seq[rs] &&
+           s_pos[re] == s_pos[re - 1] + 1)
+      ++re;
+    const bool mine = valid && i >= rs && i < re;
+    const int* table = block_tables + (size_t)s_seq[rs] * max_blocks;
+    int kmin = 0;
+    if (chunk > 0) kmin = (s_pos[rs] / chunk) * chunk;
+    if (window > 0) kmin = max(kmin, s_pos[rs] - window + 1);
+    const int kmax = s_pos[re - 1];
+
+    for (int j0 = kmin; j0 <= kmax; j0 += KT) {
+      const int nk = min(KT, kmax + 1 - j0);
+      __syncthreads();  // the previous tile is fully consumed
+      for (int e = tid; e < nk * G * DP; e += blockDim.x) {
+        const int d = e % DP, g = (e / DP) % G, jj = e / (DP * G);
+        const int j = j0 + jj;
+        const int64_t base = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+        sK[e] = d < D ? MxElem<T>::ld(kc + base * D + d) : 0.f;
+        sV[e] = d < DV ? MxElem<T>::ld(vc + base * DV + d) : 0.f;
+      }
+      __syncthreads();
+      if (mine) {
+        for (int jj = 0; jj < nk; ++jj) {
+          const float4* kr = (const float4*)(sK + (jj * G + gk) * DP);
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+          for (int d4 = 0; d4 < DP / 4; ++d4) {
+            const float4 kk = kr[d4];
+            a0 += qv[4 * d4 + 0] * kk.x;
+            a1 += qv[4 * d4 + 1] * kk.y;
+            a2 += qv[4 * d4 + 2] * kk.z;
+            a3 += qv[4 * d4 + 3] * kk.w;
+          }
+          sS[jj * NP + tid] = ((a0 + a1) + (a2 + a3)) * scale;
+        }
+      }
+      __syncthreads();
+      if (mine) {
+        float mx = m;
+        for (int jj = 0; jj < nk; ++jj) {
+          float sc;
+          if (talk != nullptr) {
+            sc = 0.f;
+            const float* tr = sT + h * H;
+            const float* sr = sS + jj * NP + i;
+            for (int g2 = 0; g2 < H; ++g2) sc += tr[g2] * sr[g2 * QT];
+          } else {
+            sc = sS[jj * NP + tid];
+          }
+          const int j = j0 + jj;
+          if (j > my_pos || j < my_lo) sc = PS_NEG_INF;
+          sM[jj * NP + tid] = sc;
+          mx = fmaxf(mx, sc);
+        }
+        if (mx > PS_NEG_INF) {
+          const float alpha = expf(m - mx);  // m = -inf gives 0
+          if (alpha != 1.f) {
+            l *= alpha;
+#pragma unroll
+            for (int d = 0; d < DP; ++d) acc[d] *= alpha;
+          }
+          m = mx;
+          for (int jj = 0; jj < nk; ++jj) {
+            const float sc = sM[jj * NP + tid];
+            if (sc > PS_NEG_INF) {
+              const float p = expf(sc - mx);
+              l += p;
+              const float4* vr = (const float4*)(sV + (jj * G + gk) * DP);
+#pragma unroll
+              for (int d4 = 0; d4 < DP / 4; ++d4) {
+                const float4 vv = vr[d4];
+                acc[4 * d4 + 0] += p * vv.x;
+                acc[4 * d4 + 1] += p * vv.y;
+                acc[4 * d4 + 2] += p * vv.z;
+                acc[4 * d4 + 3] += p * vv.w;
+              }
+            }
+          }
+        }
+      }
+    }
+    rs = re;
+  }
+  if (valid) {
+    const float inv = 1.0f / l;
+    T* o = out + (size_t)(row0 + i) * ldout + h * DV;
+#pragma unroll
+    for (int d = 0; d < DP; ++d)
+      if (d < DV) MxElem<T>::st(o + d, acc[d] * inv);
+  }
+}
+
+template <typename T, int DP>
+static int launch_tiled(void* out, int ldout, const void* q, int ldq,
+                        const void* kc, const void* vc,
+                        const void* block_tables, int max_blocks,
+                        const void* token_seq, const void* token_pos,
+                        const void* talk, int T_, int H, int G, int D, int DV,
+                        int BS, float scale, int chunk, int window, int sink,
+                        hipStream_t stream) {
+  static const size_t budget =
+      ta_lds_budget((const void*)talk_attn_tiled_kernel<T, DP>);
+  const int QT = 256 / H, NP = H * QT;
+  int KT = 32;
+  size_t lds = 0;
+  for (; KT >= 1; KT >>= 1) {
+    lds = ((size_t)2 * KT * G * DP + (size_t)2 * KT * NP + (size_t)H * H +
+           2 * QT) * sizeof(float);
+    if (lds <= budget) break;
+  }
+  if (KT < 1) return 1;
+  hipLaunchKernelGGL((talk_attn_tiled_kernel<T, DP>),
+                     dim3((T_ + QT - 1) / QT), dim3(256), lds, stream,
+                     (T*)out, ldout, (const T*)q, ldq, (const T*)kc,
+                     (const T*)vc, (const int*)block_tables, max_blocks,
+                     (const int*)token_seq, (const int*)token_pos,
+                     (const float*)talk, T_, H, G, D, DV, BS, scale, chunk,
+                     window, sink, QT, KT);
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Split-key variant for single tokens (decode): one workgroup per token,
+// thread (h, i) owns head h and key slice i of NS = 256 / H slices. Every
+// tile stages NS * KPT keys (all kv heads, fp32, rows padded against bank
+// conflicts) into LDS; thread (h, i) scores key c * NS + i of the tile for
+// its head, the heads' raw scores meet in LDS for the mix, and each thread
+// runs its own online softmax over its keys with the output accumulator in
+// registers. The NS partial results of a head are merged at the end. The
+// sink belongs to slice 0.
+template <typename T, int DP>
+__global__ __launch_bounds__(256) void talk_attn_split_kernel(
+    T* __restrict__ out, int ldout, const T* __restrict__ q, int ldq,
+    const T* __restrict__ kc, const T* __restrict__ vc,
+    const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ token_seq, const int* __restrict__ token_pos,
+    const float* __restrict__ talk, int H, int G, int D, int DV, int BS,
+    float scale, int chunk, int window, int sink, int NS, int KPT) {
+  extern __shared__ float lds[];
+  constexpr int PITCH = DP + 4;
+  const int TK = NS * KPT;           // keys per tile
+  float* sK = lds;                   // [TK][G][PITCH]
+  float* sV = sK + TK * G * PITCH;   // [TK][G][PITCH]
+  float* sS = sV + TK * G * PITCH;   // [TK][H] raw scores
+  float* sT = sS + TK * H;           // [H*H]
+  float* sML = sT + H * H;           // [2][H*NS] partial max / denominator
+  // the merge buffer [H][DP] reuses sK after the key loop
+
+  const int tid = threadIdx.x;
+  const int t = blockIdx.x;
+  const int h = tid / NS, i = tid % NS;
+  const bool valid = tid < H * NS;
+  const int rep = H / G;
+  const int gk = valid ? h / rep : 0;
+  const int pos = token_pos[t];
+  const int* table = block_tables + (size_t)token_seq[t] * max_blocks;
+  int lo = 0;
+  if (chunk > 0) lo = (pos / chunk) * chunk;
+  if (window > 0) lo = max(lo, pos - window + 1);
+
+  if (talk != nullptr)
+    for (int c = tid; c < H * H; c += blockDim.x) sT[c] = talk[c];
+  float qv[DP], acc[DP];
+#pragma unroll
+  for (int d = 0; d < DP; ++d) {
+    qv[d] = (valid && d < D)
+                ? MxElem<T>::ld(q + (size_t)t * ldq + h * D + d)
+                : 0.f;
+    acc[d] = 0.f;
+  }
+  float m = (sink && i == 0) ? 0.f : PS_NEG_INF;
+  float l = (sink && i == 0) ? 1.f : 0.f;
+
+  for (int j0 = lo; j0 <= pos; j0 += TK) {
+    const int nk = min(TK, pos + 1 - j0);
+    __syncthreads();
+    for (int e = tid; e < nk * G * DP; e += blockDim.x) {
+      const int d = e % DP, g = (e / DP) % G, jj = e / (DP * G);
+      const int j = j0 + jj;
+      const int64_t base = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+      const int o = (jj * G + g) * PITCH + d;
+      sK[o] = d < D ? MxElem<T>::ld(kc + base * D + d) : 0.f;
+      sV[o] = d < DV ? MxElem<T>::ld(vc + base * DV + d) : 0.f;
+    }
+    __syncthreads();
+    if (valid) {
+      for (int c = 0; c < KPT; ++c) {
+        const int jj = c * NS + i;
+        if (jj < nk) {
+          const float4* kr = (const float4*)(sK + (jj * G + gk) * PITCH);
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+          for (int d4 = 0; d4 < DP / 4; ++d4) {
+            const float4 kk = kr[d4];
+            a0 += qv[4 * d4 + 0] * kk.x;
+            a1 += qv[4 * d4 + 1] * kk.y;
+            a2 += qv[4 * d4 + 2] * kk.z;
+            a3 += qv[4 * d4 + 3] * kk.w;
+          }
+          sS[jj * H + h] = ((a0 + a1) + (a2 + a3)) * scale;
+        }
+      }
+    }
+    __syncthreads();
+    if (valid) {
+      for (int c = 0; c < KPT; ++c) {
+        const int jj = c * NS + i;
+        if (jj < nk) {
+          float sc;
+          if (talk != nullptr) {
+            sc = 0.f;
+            const float* tr = sT + h * H;
+            const float* sr = sS + jj * H;
+            for (int g2 = 0; g2 < H; ++g2) sc += tr[g2] * sr[g2];
+          } else {
+            sc = sS[jj * H + h];
+          }
+          const float mx = fmaxf(m, sc);
+          const float alpha = expf(m - mx);  // m = -inf gives 0
+          const float p = expf(sc - mx);
+          l = l * alpha + p;
+          m = mx;
+          const float4* vr = (const float4*)(sV + (jj * G + gk) * PITCH);
+#pragma unroll
+          for (int d4 = 0; d4 < DP / 4; ++d4) {
+            const float4 vv = vr[d4];
+            acc[4 * d4 + 0] = acc[4 * d4 + 0] * alpha + p * vv.x;
+            acc[4 * d4 + 1] = acc[4 * d4 + 1] * alpha + p * vv.y;
+            acc[4 * d4 + 2] = acc[4 * d4 + 2] * alpha + p * vv.z;
+            acc[4 * d4 + 3] = acc[4 * d4 + 3] * alpha + p * vv.w;
+          }
+        }
+      }
+    }
+  }
+  // merge the NS slices of each head
+  __syncthreads();
+  float* sOut = sK;  // [H][DP]
+  if (valid) {
+    sML[tid] = m;
+    sML[H * NS + tid] = l;
+  }
+  for (int c = tid; c < H * DP; c += blockDim.x) sOut[c] = 0.f;
+  __syncthreads();
+  float w = 0.f;
+  if (valid) {
+    float mh = PS_NEG_INF;
+    for (int r = 0; r < NS; ++r) mh = fmaxf(mh, sML[h * NS + r]);
+    float lh = 0.f;
+    for (int r = 0; r < NS; ++r) {
+      const float mr = sML[h * NS + r];
+      if (mr > PS_NEG_INF) lh += sML[H * NS + h * NS + r] * expf(mr - mh);
+    }
+    if (m > PS_NEG_INF) w = expf(m - mh) / lh;
+  }
+  for (int r = 0; r < NS; ++r) {
+    if (valid && i == r && w != 0.f) {
+#pragma unroll
+      for (int d = 0; d < DP; ++d) sOut[h * DP + d] += acc[d] * w;
+    }
+    __syncthreads();
+  }
+  for (int c = tid; c < H * DV; c += blockDim.x) {
+    const int hh = c / DV, d = c % DV;
+    MxElem<T>::st(out + (size_t)t * ldout + c, sOut[hh * DP + d]);
+  }
+}
+
+template <typename T, int DP>
+static int launch_split(void* out, int ldout, const void* q, int ldq,
+                        const void* kc, const void* vc,
+                        const void* block_tables, int max_blocks,
+                        const void* token_seq, const void* token_pos,
+                        const void* talk, int T_, int H, int G, int D, int DV,
+                        int BS, float scale, int chunk, int window, int sink,
+                        hipStream_t stream) {
+  static const size_t budget =
+      ta_lds_budget((const void*)talk_attn_split_kernel<T, DP>);
+  int NS = 0, KPT = 0;
+  size_t lds = 0;
+  // most slices first (threads), then most keys per tile (fewer barriers)
+  for (int ns = 256 / H; ns >= 1 && KPT == 0; ns >>= 1) {
+    const size_t fixed = (size_t)H * H + 2 * H * ns;
+    for (int k = 8; k >= 1; k >>= 1) {
+      const size_t tk = (size_t)ns * k;
+      size_t tile = 2 * tk * G * (DP + 4);
+      if (tile < (size_t)H * DP) tile = (size_t)H * DP;  // merge buffer
+      lds = (tile + tk * H + fixed) * sizeof(float);
+      if (lds <= budget) {
+        NS = ns;
+        KPT = k;
+        break;
+      }
+    }
+  }
+  if (KPT == 0) return 1;
+  hipLaunchKernelGGL((talk_attn_split_kernel<T, DP>), dim3(T_), dim3(256),
+                     lds, stream, (T*)out, ldout, (const T*)q, ldq,
+                     (const T*)kc, (const T*)vc, (const int*)block_tables,
+                     max_blocks, (const int*)token_seq,
+                     (const int*)token_pos, (const float*)talk, H, G, D, DV,
+                     BS, scale, chunk, window, sink, NS, KPT);
+  return 0;
+}
+
+#define TA_BY_WIDTH(FN, rc)                                                  \
+  MX_DISPATCH_DTYPE(dtype, {                                                 \
+    if (dmax <= 32)                                                          \
+      rc = FN<T, 32>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
+                     token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
+                     chunk, window, sink, (hipStream_t)stream);              \
+    else if (dmax <= 64)                                                     \
+      rc = FN<T, 64>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
+                     token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
+                     chunk, window, sink, (hipStream_t)stream);              \
+    else                                                                     \
+      rc = FN<T, 128>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,  \
+                      token_seq, token_pos, talk, T_, H, G, D, DV, BS,       \
+                      scale, chunk, window, sink, (hipStream_t)stream);      \
+  })
+
+// variant: 0 = pick for prompt portions (tiled where it fits), 3 = pick for
+// single tokens (split-key where it fits), 1 = plain one-workgroup-per-token
+// kernel, 2 = tiled only, 4 = split-key only
 extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                                  int ldq, const void* kc, const void* vc,
                                  const void* block_tables, int max_blocks,
@@ -123,8 +523,21 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                                  const void* token_pos, const void* talk,
                                  int T_, int H, int G, int D, int DV, int BS,
                                  float scale, int chunk, int window,
-                                 int sink, int dtype, void* stream) {
+                                 int sink, int dtype, int variant,
+                                 void* stream) {
   if (T_ <= 0) return 0;
+  const int dmax = D > DV ? D : DV;
+  if ((variant == 0 || variant == 2) && H <= 256 && dmax <= 128) {
+    int rc = 1;
+    TA_BY_WIDTH(launch_tiled, rc)
+    if (rc == 0) return 0;
+  }
+  if ((variant == 3 || variant == 4) && H <= 256 && dmax <= 128) {
+    int rc = 1;
+    TA_BY_WIDTH(launch_split, rc)
+    if (rc == 0) return 0;
+  }
+  if (variant == 2 || variant == 4) return 2;
   const size_t lds =
       (size_t)(H * D + 2 * H * TA_KT + H * DV + 3 * H + H * H) *
       sizeof(float);

@@ -78,10 +78,23 @@ class TalkAttention(nn.Module):
         v = proj[:, H * D + G * D:]
         ops.kv_append(k, v, k_cache, v_cache, meta.slot_mapping)
         sp = self.spec
-        return ops.talk_attention(
-            q, k_cache, v_cache, meta.block_tables, meta.token_seq,
-            meta.positions, self.scale, H, chunk=sp.chunk, window=sp.window,
-            sink=sp.sink, talk=self.talk, out=out)
+        T = proj.shape[0]
+        if out is None:
+            out = torch.empty((T, H * DV), dtype=proj.dtype,
+                              device=proj.device)
+        # batch rows: multi-token prompt portions first, single tokens
+        # after them. Portions share key tiles between neighbouring rows
+        # (tiled kernel); single tokens of different sequences share
+        # nothing and take the split-key kernel, one workgroup per token.
+        npt = min(getattr(meta, "num_prefill_tokens", T) or 0, T)
+        for a, b, variant in ((0, npt, 0), (npt, T, 3)):
+            if b > a:
+                ops.talk_attention(
+                    q[a:b], k_cache, v_cache, meta.block_tables,
+                    meta.token_seq[a:b], meta.positions[a:b], self.scale, H,
+                    chunk=sp.chunk, window=sp.window, sink=sp.sink,
+                    talk=self.talk, out=out[a:b], variant=variant)
+        return out
 
 
 class GeneralDelta(nn.Module):

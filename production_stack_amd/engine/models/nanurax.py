@@ -242,19 +242,18 @@ class NanuraxForCausalLM(nn.Module):
     # ---- weights -------------------------------------------------------
     @torch.no_grad()
     def random_init(self, seed: int = 0) -> None:
-        gen = torch.Generator(device="cpu").manual_seed(seed)
+        dev = self.embed.device
+        gen = torch.Generator(device=dev).manual_seed(seed)
         for name, p in self.named_parameters():
-            if name.endswith("norm") or name.endswith("out_norm"):
-                v = 1.0 + 0.1 * torch.randn(p.shape, generator=gen)
+            if name.endswith("norm"):
+                p.normal_(1.0, 0.1, generator=gen)
             elif name.endswith(("w0", "a_bias")):
-                v = 0.5 * torch.randn(p.shape, generator=gen)
+                p.normal_(0.0, 0.5, generator=gen)
             elif name.endswith("talk"):
-                v = torch.eye(p.shape[0]) + 0.2 * torch.randn(
-                    p.shape, generator=gen)
+                p.normal_(0.0, 0.2, generator=gen)
+                p.add_(torch.eye(p.shape[0], device=dev, dtype=p.dtype))
             else:
-                fan_in = p.shape[-1]
-                v = torch.randn(p.shape, generator=gen) / fan_in ** 0.5
-            p.copy_(v.to(p.dtype))
+                p.normal_(0.0, p.shape[-1] ** -0.5, generator=gen)
         for layer in self.layers:
             layer.w_in = layer.w_out = None
 

@@ -540,11 +540,16 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
                    token_seq: torch.Tensor, token_pos: torch.Tensor,
                    scale: float, heads: int, chunk: int = 0, window: int = 0,
                    sink: bool = False, talk: torch.Tensor = None,
-                   out: torch.Tensor = None) -> torch.Tensor:
+                   out: torch.Tensor = None, variant: int = 0
+                   ) -> torch.Tensor:
     """Paged attention of a ragged batch. q [T, H*D] (row-strided view
     allowed); token_seq/token_pos int32 [T] give each token's block-table
     row and position; talk: optional fp32 [H, H] score mix; chunk/window:
     visibility limits (0 = off); sink: add 1 to the softmax denominator.
+    variant 0 picks the kernel for prompt portions (tiled thread-per-
+    (head, query) where the shape fits), 3 for single tokens (split-key),
+    both falling back to the plain one-workgroup-per-token kernel; 1 / 2 /
+    4 force plain / tiled / split-key.
     Returns [T, H*DV]."""
     NB, G, BS, D = k_cache.shape
     DV = v_cache.shape[3]
@@ -574,7 +579,7 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
         _p(v_cache), _p(block_tables), block_tables.shape[1],
         _p(token_seq), _p(token_pos), _p(talk), T, H, G, D, DV, BS,
         _f(scale), int(chunk), int(window), int(bool(sink)),
-        _mx_dtype(q.dtype), _stream())
+        _mx_dtype(q.dtype), int(variant), _stream())
     if rc != 0:
         raise RuntimeError(
             f"talk_attention: heads x dim {H}x{D}/{DV} exceeds the kernel's "

@@ -105,14 +105,19 @@ def test_kv_append_distinct_widths(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("variant", [1, 2, 4])
 @pytest.mark.parametrize("H,G,D,DV,chunk,window,sink,talk", [
     (4, 2, 40, 40, 24, 0, True, True),
     (6, 3, 40, 24, 40, 0, True, True),
     (3, 1, 32, 64, 0, 0, False, False),
     (4, 4, 16, 16, 0, 20, True, False),
     (8, 2, 64, 32, 37, 0, False, True),
+    (32, 8, 128, 128, 64, 0, True, True),
+    (16, 4, 72, 96, 0, 50, True, True),
+    (5, 5, 24, 24, 30, 0, True, True),
 ])
-def test_talk_attention(dtype, H, G, D, DV, chunk, window, sink, talk):
+def test_talk_attention(dtype, variant, H, G, D, DV, chunk, window, sink,
+                        talk):
     g = torch.Generator().manual_seed(4)
     bs, n_seqs, L = 16, 3, 150
     kc, vc, tables = _paged(L, G, D, DV, bs, dtype, g, n_seqs)
@@ -125,6 +130,10 @@ def test_talk_attention(dtype, H, G, D, DV, chunk, window, sink, talk):
     edge = chunk or window or bs
     for p in (edge - 1, edge, edge + 1, 2 * edge - 1, 2 * edge):
         token_seq.append(1)
+        token_pos.append(p)
+    # single tokens of different sequences side by side (decode rows)
+    for s, p in ((0, 69), (2, 149), (1, 130), (2, 0), (0, 0), (1, 1)):
+        token_seq.append(s)
         token_pos.append(p)
     T = len(token_seq)
     q = torch.randn(T, H * D + 5, generator=g).to(dtype)
@@ -139,7 +148,7 @@ def test_talk_attention(dtype, H, G, D, DV, chunk, window, sink, talk):
     got = ops.talk_attention(
         q.cuda()[:, :H * D], kc.cuda(), vc.cuda(), tables.cuda(), ts.cuda(),
         tp.cuda(), scale, H, chunk=chunk, window=window, sink=sink,
-        talk=tk.cuda() if tk is not None else None)
+        talk=tk.cuda() if tk is not None else None, variant=variant)
     torch.testing.assert_close(got.cpu().float().view(T, H, DV), want,
                                **tol(dtype))
 

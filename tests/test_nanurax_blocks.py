@@ -132,6 +132,16 @@ class Harness:
         """parts: [(seq index, first position, projections [n, rows])];
         returns the mixer's outputs, one tensor per part."""
         bs, dev = self.bs, self.device
+        # the runner's batch order: multi-token portions, then single tokens
+        order = sorted(range(len(parts)),
+                       key=lambda i: parts[i][2].shape[0] == 1)
+        if order != list(range(len(parts))):
+            res = self.run([parts[i] for i in order], slot_of)
+            back = [None] * len(parts)
+            for k, i in enumerate(order):
+                back[i] = res[k]
+            return back
+        n_multi = sum(p.shape[0] for _, _, p in parts if p.shape[0] > 1)
         proj = torch.cat([p for _, _, p in parts]).to(dev)
         pos, tseq, slots, rows = [], [], [], []
         r0 = 0
@@ -147,7 +157,7 @@ class Harness:
         meta = BatchMeta(
             positions=torch.tensor(pos, dtype=torch.int32, device=dev),
             slot_mapping=torch.tensor(slots, dtype=torch.long, device=dev),
-            num_prefill_tokens=0, prefill_token_seq=None,
+            num_prefill_tokens=n_multi, prefill_token_seq=None,
             prefill_token_pos=None, prefill_block_tables=None,
             num_decode_seqs=0, decode_seq_lens=None,
             decode_block_tables=None,
