@@ -128,6 +128,86 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
     MxElem<T>::st(out + (size_t)t * ldout + it, sacc[it] / sl[it / DV]);
 }
 
+// Stage nk keys x G kv heads of one cache (rows of Dw elements) into LDS as
+// fp32 rows of PITCH floats, columns [Dw, DP) zeroed. Rows are read with
+// 16-byte loads, several in flight per thread before any is consumed (the
+// kernels run one wave per SIMD, so nothing else hides the latency).
+template <typename T>
+struct TaVec;
+template <>
+struct TaVec<float> {
+  static constexpr int N = 4;
+  static PS_DEV void put(float* dst, const float4& v) {
+    *(float4*)dst = v;
+  }
+};
+template <>
+struct TaVec<mx_bf16> {
+  static constexpr int N = 8;
+  static PS_DEV void put(float* dst, const float4& v) {
+    const unsigned int* u = (const unsigned int*)&v;
+    float4 a, b;
+    a.x = __uint_as_float(u[0] << 16);
+    a.y = __uint_as_float(u[0] & 0xffff0000u);
+    a.z = __uint_as_float(u[1] << 16);
+    a.w = __uint_as_float(u[1] & 0xffff0000u);
+    b.x = __uint_as_float(u[2] << 16);
+    b.y = __uint_as_float(u[2] & 0xffff0000u);
+    b.z = __uint_as_float(u[3] << 16);
+    b.w = __uint_as_float(u[3] & 0xffff0000u);
+    *(float4*)dst = a;
+    *(float4*)(dst + 4) = b;
+  }
+};
+
+template <typename T, int DP, int PITCH>
+PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
+                     const int* __restrict__ table, int j0, int nk, int G,
+                     int Dw, int BS) {
+  constexpr int VEC = TaVec<T>::N;
+  constexpr int U = 4;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  if (Dw % VEC == 0) {
+    const int vpr = Dw / VEC;
+    const int total = nk * G * vpr;
+    for (int base = 0; base < total; base += nt * U) {
+      float4 buf[U];
+      int off[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int idx = base + u * nt + tid;
+        off[u] = -1;
+        if (idx < total) {
+          const int row = idx / vpr, c = idx - row * vpr;
+          const int jj = row / G, g = row - jj * G;
+          const int j = j0 + jj;
+          const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+          buf[u] = *(const float4*)(cache + gb * Dw + c * VEC);
+          off[u] = row * PITCH + c * VEC;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (off[u] >= 0) TaVec<T>::put(sdst + off[u], buf[u]);
+    }
+    if (Dw < DP) {
+      const int pad = DP - Dw;
+      for (int e = tid; e < nk * G * pad; e += nt) {
+        const int row = e / pad, d = Dw + e - row * pad;
+        sdst[row * PITCH + d] = 0.f;
+      }
+    }
+  } else {
+    for (int e = tid; e < nk * G * DP; e += nt) {
+      const int d = e % DP, row = e / DP;
+      const int jj = row / G, g = row - jj * G;
+      const int j = j0 + jj;
+      const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+      sdst[row * PITCH + d] = d < Dw ? MxElem<T>::ld(cache + gb * Dw + d) : 0.f;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Tiled variant: one thread per (head, query) pair.
 //
@@ -205,13 +285,8 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
     for (int j0 = kmin; j0 <= kmax; j0 += KT) {
       const int nk = min(KT, kmax + 1 - j0);
       __syncthreads();  // the previous tile is fully consumed
-      for (int e = tid; e < nk * G * DP; e += blockDim.x) {
-        const int d = e % DP, g = (e / DP) % G, jj = e / (DP * G);
-        const int j = j0 + jj;
-        const int64_t base = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-        sK[e] = d < D ? MxElem<T>::ld(kc + base * D + d) : 0.f;
-        sV[e] = d < DV ? MxElem<T>::ld(vc + base * DV + d) : 0.f;
-      }
+      ta_stage<T, DP, DP>(sK, kc, table, j0, nk, G, D, BS);
+      ta_stage<T, DP, DP>(sV, vc, table, j0, nk, G, DV, BS);
       __syncthreads();
       if (mine) {
         for (int jj = 0; jj < nk; ++jj) {
@@ -368,14 +443,8 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   for (int j0 = lo; j0 <= pos; j0 += TK) {
     const int nk = min(TK, pos + 1 - j0);
     __syncthreads();
-    for (int e = tid; e < nk * G * DP; e += blockDim.x) {
-      const int d = e % DP, g = (e / DP) % G, jj = e / (DP * G);
-      const int j = j0 + jj;
-      const int64_t base = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-      const int o = (jj * G + g) * PITCH + d;
-      sK[o] = d < D ? MxElem<T>::ld(kc + base * D + d) : 0.f;
-      sV[o] = d < DV ? MxElem<T>::ld(vc + base * DV + d) : 0.f;
-    }
+    ta_stage<T, DP, PITCH>(sK, kc, table, j0, nk, G, D, BS);
+    ta_stage<T, DP, PITCH>(sV, vc, table, j0, nk, G, DV, BS);
     __syncthreads();
     if (valid) {
       for (int c = 0; c < KPT; ++c) {
