@@ -11,16 +11,20 @@
 // and the head's o is divided by its root mean square, scaled by a channel
 // weight and by sigmoid(g).
 //
-// Mapping: one workgroup per (sequence segment, head); thread j owns column
-// j of S in registers (DKP rows, D padded up), so u^T S and S^T r are
-// thread-local dot products and the only cross-lane traffic is the two
-// norms. Tokens go through in tiles: the per-row vectors (u, a*u, w, k, r)
-// of a whole tile are prepared cooperatively into LDS, then each thread
-// walks the tile's tokens with broadcast LDS reads and no barrier.
+// Mapping: one workgroup per (sequence segment, head). Column j of S lives
+// in the registers of P adjacent lanes, lane p holding rows p, p+P, ...
+// (DKP / P rows, D padded up to DKP), so u^T S and S^T r are short
+// thread-local dot products finished by a P-lane butterfly; the only other
+// cross-lane traffic is the two norms. Tokens go through in tiles: the
+// per-row vectors (u, a*u, w, k, r) of a whole tile are prepared
+// cooperatively into LDS (stored so that each lane's rows are contiguous),
+// then each thread walks the tile's tokens with broadcast LDS reads and no
+// barrier.
 #include "mix_common.h"
 
-template <typename T, int DKP, int TILE>
-__global__ __launch_bounds__(256) void delta_rule_kernel(
+template <typename T, int DKP, int TILE, int P>
+__global__ __launch_bounds__(DKP * P <= 256 ? 256 : DKP * P)
+void delta_rule_kernel(
     T* __restrict__ out, int ldo, const T* __restrict__ r, int ldr,
     const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const T* __restrict__ zw, int ldzw, const T* __restrict__ za, int ldza,
@@ -34,22 +38,25 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   float* sw = sau + TILE * DKP;     // decay
   float* sk = sw + TILE * DKP;      // key
   float* sr = sk + TILE * DKP;      // receptance
-  float* red = sr + TILE * DKP;     // [4][TILE] cross-wave partials
+  float* red = sr + TILE * DKP;     // [16][TILE] cross-wave partials
+  constexpr int R = DKP / P;        // rows per lane
 
   const int seg = blockIdx.x / H, hd = blockIdx.x % H;
   const int t0 = seq_rows[4 * seg + 0], n = seq_rows[4 * seg + 1];
   const int p0 = seq_rows[4 * seg + 2], slot = seq_rows[4 * seg + 3];
-  const int j = threadIdx.x;
+  const int j = threadIdx.x / P, p = threadIdx.x % P;
   const bool col = j < D;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   const int hc = hd * D;  // channel offset of this head
 
   float* Sg = state + ((size_t)slot * H + hd) * (size_t)D * D;
-  float S[DKP];
+  float S[R];  // S[k] = row p + P * k of column j
 #pragma unroll
-  for (int i = 0; i < DKP; ++i)
-    S[i] = (col && i < D && p0 != 0) ? Sg[(size_t)i * D + j] : 0.f;
+  for (int k2 = 0; k2 < R; ++k2) {
+    const int i = p + P * k2;
+    S[k2] = (col && i < D && p0 != 0) ? Sg[(size_t)i * D + j] : 0.f;
+  }
 
   for (int tb = 0; tb < n; tb += TILE) {
     const int nt = min(TILE, n - tb);
@@ -66,10 +73,12 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
         wv = expf(-decay_scale * mx_sigmoid(z));
         av = mx_sigmoid(MxElem<T>::ld(za + row * ldza + c) + ab[c]);
       }
-      sk[idx] = kv;
-      sr[idx] = rv;
-      sw[idx] = wv;
-      sau[idx] = av;
+      // row i is kept at (i % P) * R + i / P: a lane's rows are contiguous
+      const int at = tt * DKP + (i % P) * R + i / P;
+      sk[at] = kv;
+      sr[at] = rv;
+      sw[at] = wv;
+      sau[at] = av;
     }
     __syncthreads();
     for (int tt = wave; tt < nt; tt += nw) {
@@ -95,21 +104,25 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
       if (tt < nt) {
         const size_t row = (size_t)(t0 + tb + tt);
         const float vj = col ? MxElem<T>::ld(v + row * ldv + hc + j) : 0.f;
-        const float* pu = su + tt * DKP;
-        const float* pau = sau + tt * DKP;
-        const float* pw = sw + tt * DKP;
-        const float* pk = sk + tt * DKP;
-        const float* pr = sr + tt * DKP;
+        const float* pu = su + tt * DKP + p * R;
+        const float* pau = sau + tt * DKP + p * R;
+        const float* pw = sw + tt * DKP + p * R;
+        const float* pk = sk + tt * DKP + p * R;
+        const float* pr = sr + tt * DKP + p * R;
         float sa = 0.f;
 #pragma unroll
-        for (int i = 0; i < DKP; ++i) sa += pu[i] * S[i];
+        for (int i = 0; i < R; ++i) sa += pu[i] * S[i];
+#pragma unroll
+        for (int off = 1; off < P; off <<= 1) sa += __shfl_xor(sa, off, 64);
         float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < DKP; ++i) {
+        for (int i = 0; i < R; ++i) {
           const float s = pw[i] * S[i] - pau[i] * sa + pk[i] * vj;
           S[i] = s;
           acc += s * pr[i];
         }
+#pragma unroll
+        for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, 64);
         o[tt] = acc;
       }
     }
@@ -117,11 +130,11 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     // per-token sum over the head's columns of o^2
 #pragma unroll
     for (int tt = 0; tt < TILE; ++tt) {
-      const float q = mx_wave_sum(col ? o[tt] * o[tt] : 0.f);
+      const float q = mx_wave_sum((col && p == 0) ? o[tt] * o[tt] : 0.f);
       if (lane == 0) red[wave * TILE + tt] = q;
     }
     __syncthreads();
-    if (col) {
+    if (col && p == 0) {
 #pragma unroll
       for (int tt = 0; tt < TILE; ++tt) {
         if (tt < nt) {
@@ -139,8 +152,10 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   }
   if (col) {
 #pragma unroll
-    for (int i = 0; i < DKP; ++i)
-      if (i < D) Sg[(size_t)i * D + j] = S[i];
+    for (int k2 = 0; k2 < R; ++k2) {
+      const int i = p + P * k2;
+      if (i < D) Sg[(size_t)i * D + j] = S[k2];
+    }
   }
 }
 
@@ -153,9 +168,10 @@ static void launch_delta(void* out, int ldo, const void* r, int ldr,
                          const void* seq_rows, int S_, int H, int D,
                          float eps, float decay_scale, hipStream_t stream) {
   constexpr int TILE = DKP <= 128 ? 16 : 8;
-  const int threads = ((D + 63) / 64) * 64;
-  const size_t lds = (size_t)(5 * TILE * DKP + 4 * TILE) * sizeof(float);
-  hipLaunchKernelGGL((delta_rule_kernel<T, DKP, TILE>), dim3(S_ * H),
+  constexpr int P = DKP >= 64 ? 4 : (DKP >= 32 ? 2 : 1);
+  const int threads = ((D * P + 63) / 64) * 64;
+  const size_t lds = (size_t)(5 * TILE * DKP + 16 * TILE) * sizeof(float);
+  hipLaunchKernelGGL((delta_rule_kernel<T, DKP, TILE, P>), dim3(S_ * H),
                      dim3(threads), lds, stream, (T*)out, ldo, (const T*)r,
                      ldr, (const T*)k, ldk, (const T*)v, ldv, (const T*)zw,
                      ldzw, (const T*)za, ldza, (const T*)g, ldg,
