@@ -32,14 +32,19 @@ void delta_rule_kernel(
     const float* __restrict__ ab, const float* __restrict__ normw,
     float* __restrict__ state, const int* __restrict__ seq_rows, int H, int D,
     float eps, float decay_scale) {
-  extern __shared__ float lds[];
-  float* su = lds;                  // [TILE][DKP] unit key
-  float* sau = su + TILE * DKP;     // a * u
-  float* sw = sau + TILE * DKP;     // decay
-  float* sk = sw + TILE * DKP;      // key
-  float* sr = sk + TILE * DKP;      // receptance
-  float* red = sr + TILE * DKP;     // [16][TILE] cross-wave partials
+  extern __shared__ __align__(16) float lds[];
   constexpr int R = DKP / P;        // rows per lane
+  // a lane's R rows are contiguous; the P segments of a token are RP words
+  // apart so that the P addresses of one broadcast read fall into
+  // different banks
+  constexpr int RP = P > 1 ? R + 4 : R;
+  constexpr int TP = RP * P;        // words per token and array
+  float* su = lds;                  // [TILE][TP] unit key
+  float* sau = su + TILE * TP;      // a * u
+  float* sw = sau + TILE * TP;      // decay
+  float* sk = sw + TILE * TP;       // key
+  float* sr = sk + TILE * TP;       // receptance
+  float* red = sr + TILE * TP;      // [16][TILE] cross-wave partials
 
   const int seg = blockIdx.x / H, hd = blockIdx.x % H;
   const int t0 = seq_rows[4 * seg + 0], n = seq_rows[4 * seg + 1];
@@ -61,38 +66,70 @@ void delta_rule_kernel(
   for (int tb = 0; tb < n; tb += TILE) {
     const int nt = min(TILE, n - tb);
     __syncthreads();  // previous tile's LDS reads are done
-    for (int idx = threadIdx.x; idx < nt * DKP; idx += blockDim.x) {
-      const int tt = idx / DKP, i = idx % DKP;
-      float kv = 0.f, rv = 0.f, wv = 0.f, av = 0.f;
-      if (i < D) {
-        const size_t row = (size_t)(t0 + tb + tt);
-        const int c = hc + i;
-        kv = MxElem<T>::ld(k + row * ldk + c);
-        rv = MxElem<T>::ld(r + row * ldr + c);
-        const float z = MxElem<T>::ld(zw + row * ldzw + c) + w0[c];
-        wv = expf(-decay_scale * mx_sigmoid(z));
-        av = mx_sigmoid(MxElem<T>::ld(za + row * ldza + c) + ab[c]);
+    // this tile's value and gate entries of column j: issued together, up
+    // front, so their latency hides behind the cooperative preparation
+    float vreg[TILE], greg[TILE];
+#pragma unroll
+    for (int tt = 0; tt < TILE; ++tt) {
+      const size_t row = (size_t)(t0 + tb + min(tt, nt - 1));
+      vreg[tt] = col ? MxElem<T>::ld(v + row * ldv + hc + j) : 0.f;
+      greg[tt] = col ? MxElem<T>::ld(g + row * ldg + hc + j) : 0.f;
+    }
+    // four elements per thread and pass, all their loads before any use
+    for (int base = 0; base < nt * DKP; base += blockDim.x * 4) {
+      float kv[4], rv[4], zv[4], av[4];
+      int at[4], ch[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * blockDim.x + threadIdx.x;
+        at[u] = -1;
+        ch[u] = -1;
+        kv[u] = rv[u] = zv[u] = av[u] = 0.f;
+        if (idx < nt * DKP) {
+          const int tt = idx / DKP, i = idx % DKP;
+          // row i is kept at (i % P) * R + i / P: a lane's rows are
+          // contiguous
+          at[u] = tt * TP + (i % P) * RP + i / P;
+          if (i < D) {
+            const size_t row = (size_t)(t0 + tb + tt);
+            const int c = hc + i;
+            ch[u] = c;
+            kv[u] = MxElem<T>::ld(k + row * ldk + c);
+            rv[u] = MxElem<T>::ld(r + row * ldr + c);
+            zv[u] = MxElem<T>::ld(zw + row * ldzw + c);
+            av[u] = MxElem<T>::ld(za + row * ldza + c);
+          }
+        }
       }
-      // row i is kept at (i % P) * R + i / P: a lane's rows are contiguous
-      const int at = tt * DKP + (i % P) * R + i / P;
-      sk[at] = kv;
-      sr[at] = rv;
-      sw[at] = wv;
-      sau[at] = av;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (at[u] >= 0) {
+          float wv = 0.f, aa = 0.f;
+          if (ch[u] >= 0) {
+            wv = expf(-decay_scale * mx_sigmoid(zv[u] + w0[ch[u]]));
+            aa = mx_sigmoid(av[u] + ab[ch[u]]);
+          }
+          sk[at[u]] = kv[u];
+          sr[at[u]] = rv[u];
+          sw[at[u]] = wv;
+          sau[at[u]] = aa;
+        }
+      }
     }
     __syncthreads();
     for (int tt = wave; tt < nt; tt += nw) {
       float ss = 0.f;
       for (int i = lane; i < DKP; i += 64) {
-        const float kv = sk[tt * DKP + i];
+        const float kv = sk[tt * TP + (i % P) * RP + i / P];
         ss += kv * kv;
       }
       ss = mx_wave_sum(ss);
       const float inv = 1.0f / sqrtf(ss + 1e-6f);
       for (int i = lane; i < DKP; i += 64) {
-        const float u = sk[tt * DKP + i] * inv;
-        su[tt * DKP + i] = u;
-        sau[tt * DKP + i] *= u;
+        const int at = tt * TP + (i % P) * RP + i / P;
+        const float u = sk[at] * inv;
+        su[at] = u;
+        sau[at] *= u;
       }
     }
     __syncthreads();
@@ -102,24 +139,35 @@ void delta_rule_kernel(
     for (int tt = 0; tt < TILE; ++tt) {
       o[tt] = 0.f;
       if (tt < nt) {
-        const size_t row = (size_t)(t0 + tb + tt);
-        const float vj = col ? MxElem<T>::ld(v + row * ldv + hc + j) : 0.f;
-        const float* pu = su + tt * DKP + p * R;
-        const float* pau = sau + tt * DKP + p * R;
-        const float* pw = sw + tt * DKP + p * R;
-        const float* pk = sk + tt * DKP + p * R;
-        const float* pr = sr + tt * DKP + p * R;
+        const float vj = vreg[tt];
+        const float4* pu = (const float4*)(su + tt * TP + p * RP);
+        const float4* pau = (const float4*)(sau + tt * TP + p * RP);
+        const float4* pw = (const float4*)(sw + tt * TP + p * RP);
+        const float4* pk = (const float4*)(sk + tt * TP + p * RP);
+        const float4* pr = (const float4*)(sr + tt * TP + p * RP);
         float sa = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) sa += pu[i] * S[i];
+        for (int i = 0; i < R / 4; ++i) {
+          const float4 u4 = pu[i];
+          sa += u4.x * S[4 * i] + u4.y * S[4 * i + 1] + u4.z * S[4 * i + 2] +
+                u4.w * S[4 * i + 3];
+        }
 #pragma unroll
         for (int off = 1; off < P; off <<= 1) sa += __shfl_xor(sa, off, 64);
         float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-          const float s = pw[i] * S[i] - pau[i] * sa + pk[i] * vj;
-          S[i] = s;
-          acc += s * pr[i];
+        for (int i = 0; i < R / 4; ++i) {
+          const float4 w4 = pw[i], a4 = pau[i], k4 = pk[i], r4 = pr[i];
+          const float wv[4] = {w4.x, w4.y, w4.z, w4.w};
+          const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+          const float kv[4] = {k4.x, k4.y, k4.z, k4.w};
+          const float rv[4] = {r4.x, r4.y, r4.z, r4.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float s = wv[e] * S[4 * i + e] - av[e] * sa + kv[e] * vj;
+            S[4 * i + e] = s;
+            acc += s * rv[e];
+          }
         }
 #pragma unroll
         for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, 64);
@@ -142,8 +190,7 @@ void delta_rule_kernel(
           for (int w = 0; w < nw; ++w) ss += red[w * TILE + tt];
           const size_t row = (size_t)(t0 + tb + tt);
           const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-          const float gate =
-              mx_sigmoid(MxElem<T>::ld(g + row * ldg + hc + j));
+          const float gate = mx_sigmoid(greg[tt]);
           MxElem<T>::st(out + row * ldo + hc + j,
                         o[tt] * inv * normw[hc + j] * gate);
         }
@@ -170,7 +217,9 @@ static void launch_delta(void* out, int ldo, const void* r, int ldr,
   constexpr int TILE = DKP <= 128 ? 16 : 8;
   constexpr int P = DKP >= 64 ? 4 : (DKP >= 32 ? 2 : 1);
   const int threads = ((D * P + 63) / 64) * 64;
-  const size_t lds = (size_t)(5 * TILE * DKP + 16 * TILE) * sizeof(float);
+  const size_t lds =
+      (size_t)(5 * TILE * (DKP + (P > 1 ? 4 * P : 0)) + 16 * TILE) *
+      sizeof(float);
   hipLaunchKernelGGL((delta_rule_kernel<T, DKP, TILE, P>), dim3(S_ * H),
                      dim3(threads), lds, stream, (T*)out, ldo, (const T*)r,
                      ldr, (const T*)k, ldk, (const T*)v, ldv, (const T*)zw,
