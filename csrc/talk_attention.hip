@@ -404,7 +404,8 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
     const float* __restrict__ talk, int H, int G, int D, int DV, int BS,
-    float scale, int chunk, int window, int sink, int NS, int KPT) {
+    float scale, int chunk, int window, int sink, int NS, int KPT, int KS,
+    float* __restrict__ part) {
   extern __shared__ float lds[];
   constexpr int PITCH = DP + 4;
   const int TK = NS * KPT;           // keys per tile
@@ -416,16 +417,23 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   // the merge buffer [H][DP] reuses sK after the key loop
 
   const int tid = threadIdx.x;
-  const int t = blockIdx.x;
+  const int t = blockIdx.x / KS, ks = blockIdx.x % KS;
   const int h = tid / NS, i = tid % NS;
   const bool valid = tid < H * NS;
   const int rep = H / G;
   const int gk = valid ? h / rep : 0;
-  const int pos = token_pos[t];
   const int* table = block_tables + (size_t)token_seq[t] * max_blocks;
-  int lo = 0;
+  int lo = 0, pos = token_pos[t];
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
+  if (KS > 1) {
+    // this workgroup's share of the visible keys, in whole tiles
+    const int tiles = (pos + 1 - lo + TK - 1) / TK;
+    const int per = (tiles + KS - 1) / KS;
+    const int first = lo + ks * per * TK;
+    pos = min(pos, first + per * TK - 1);
+    lo = first;  // may pass pos: then this share is empty
+  }
 
   if (talk != nullptr)
     for (int c = tid; c < H * H; c += blockDim.x) sT[c] = talk[c];
@@ -437,8 +445,9 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
                 : 0.f;
     acc[d] = 0.f;
   }
-  float m = (sink && i == 0) ? 0.f : PS_NEG_INF;
-  float l = (sink && i == 0) ? 1.f : 0.f;
+  const bool own_sink = sink && i == 0 && ks == 0;
+  float m = own_sink ? 0.f : PS_NEG_INF;
+  float l = own_sink ? 1.f : 0.f;
 
   for (int j0 = lo; j0 <= pos; j0 += TK) {
     const int nk = min(TK, pos + 1 - j0);
@@ -506,15 +515,16 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   for (int c = tid; c < H * DP; c += blockDim.x) sOut[c] = 0.f;
   __syncthreads();
   float w = 0.f;
+  float mh = PS_NEG_INF, lh = 0.f;
   if (valid) {
-    float mh = PS_NEG_INF;
     for (int r = 0; r < NS; ++r) mh = fmaxf(mh, sML[h * NS + r]);
-    float lh = 0.f;
     for (int r = 0; r < NS; ++r) {
       const float mr = sML[h * NS + r];
       if (mr > PS_NEG_INF) lh += sML[H * NS + h * NS + r] * expf(mr - mh);
     }
-    if (m > PS_NEG_INF) w = expf(m - mh) / lh;
+    // one workgroup per token: normalise here; several: leave the sum
+    // relative to mh for the combine kernel
+    if (m > PS_NEG_INF) w = expf(m - mh) / (KS > 1 ? 1.f : lh);
   }
   for (int r = 0; r < NS; ++r) {
     if (valid && i == r && w != 0.f) {
@@ -523,9 +533,47 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
     }
     __syncthreads();
   }
-  for (int c = tid; c < H * DV; c += blockDim.x) {
-    const int hh = c / DV, d = c % DV;
-    MxElem<T>::st(out + (size_t)t * ldout + c, sOut[hh * DP + d]);
+  if (KS == 1) {
+    for (int c = tid; c < H * DV; c += blockDim.x) {
+      const int hh = c / DV, d = c % DV;
+      MxElem<T>::st(out + (size_t)t * ldout + c, sOut[hh * DP + d]);
+    }
+  } else {
+    // partial record per (token, share, head): max, denominator, DV sums
+    float* rec = part + ((size_t)t * KS + ks) * H * (DV + 2);
+    if (valid && i == 0) {
+      rec[h * (DV + 2)] = mh;
+      rec[h * (DV + 2) + 1] = lh;
+    }
+    for (int c = tid; c < H * DV; c += blockDim.x) {
+      const int hh = c / DV, d = c % DV;
+      rec[hh * (DV + 2) + 2 + d] = sOut[hh * DP + d];
+    }
+  }
+}
+
+// Merge the KS partial records of every (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void talk_attn_combine_kernel(
+    T* __restrict__ out, int ldout, const float* __restrict__ part, int H,
+    int DV, int KS) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < H * DV; c += blockDim.x) {
+    const int h = c / DV, d = c % DV;
+    const float* rec = part + (size_t)t * KS * H * (DV + 2) + h * (DV + 2);
+    const size_t step = (size_t)H * (DV + 2);
+    float mh = PS_NEG_INF;
+    for (int s = 0; s < KS; ++s) mh = fmaxf(mh, rec[s * step]);
+    float l = 0.f, a = 0.f;
+    for (int s = 0; s < KS; ++s) {
+      const float ms = rec[s * step];
+      if (ms > PS_NEG_INF) {
+        const float w = expf(ms - mh);
+        l += rec[s * step + 1] * w;
+        a += rec[s * step + 2 + d] * w;
+      }
+    }
+    MxElem<T>::st(out + (size_t)t * ldout + c, a / l);
   }
 }
 
@@ -536,9 +584,10 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
                         const void* token_seq, const void* token_pos,
                         const void* talk, int T_, int H, int G, int D, int DV,
                         int BS, float scale, int chunk, int window, int sink,
-                        hipStream_t stream) {
+                        hipStream_t stream, int KS, float* part) {
   static const size_t budget =
       ta_lds_budget((const void*)talk_attn_split_kernel<T, DP>);
+  if (KS < 1 || part == nullptr) KS = 1;
   int NS = 0, KPT = 0;
   size_t lds = 0;
   // most slices first (threads), then most keys per tile (fewer barriers)
@@ -557,29 +606,35 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
     }
   }
   if (KPT == 0) return 1;
-  hipLaunchKernelGGL((talk_attn_split_kernel<T, DP>), dim3(T_), dim3(256),
-                     lds, stream, (T*)out, ldout, (const T*)q, ldq,
+  hipLaunchKernelGGL((talk_attn_split_kernel<T, DP>), dim3(T_ * KS),
+                     dim3(256), lds, stream, (T*)out, ldout, (const T*)q, ldq,
                      (const T*)kc, (const T*)vc, (const int*)block_tables,
                      max_blocks, (const int*)token_seq,
                      (const int*)token_pos, (const float*)talk, H, G, D, DV,
-                     BS, scale, chunk, window, sink, NS, KPT);
+                     BS, scale, chunk, window, sink, NS, KPT, KS, part);
+  if (KS > 1)
+    hipLaunchKernelGGL((talk_attn_combine_kernel<T>), dim3(T_), dim3(256), 0,
+                       stream, (T*)out, ldout, (const float*)part, H, DV, KS);
   return 0;
 }
 
-#define TA_BY_WIDTH(FN, rc)                                                  \
+#define TA_BY_WIDTH(FN, rc, ...)                                               \
   MX_DISPATCH_DTYPE(dtype, {                                                 \
     if (dmax <= 32)                                                          \
       rc = FN<T, 32>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
                      token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
-                     chunk, window, sink, (hipStream_t)stream);              \
+                     chunk, window, sink, (hipStream_t)stream,               \
+                     ##__VA_ARGS__);                                         \
     else if (dmax <= 64)                                                     \
       rc = FN<T, 64>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
                      token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
-                     chunk, window, sink, (hipStream_t)stream);              \
+                     chunk, window, sink, (hipStream_t)stream,               \
+                     ##__VA_ARGS__);                                         \
     else                                                                     \
       rc = FN<T, 128>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,  \
                       token_seq, token_pos, talk, T_, H, G, D, DV, BS,       \
-                      scale, chunk, window, sink, (hipStream_t)stream);      \
+                      scale, chunk, window, sink, (hipStream_t)stream,       \
+                      ##__VA_ARGS__);                                        \
   })
 
 // variant: 0 = pick for prompt portions (tiled where it fits), 3 = pick for
@@ -593,7 +648,7 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                                  int T_, int H, int G, int D, int DV, int BS,
                                  float scale, int chunk, int window,
                                  int sink, int dtype, int variant,
-                                 void* stream) {
+                                 int splits, void* scratch, void* stream) {
   if (T_ <= 0) return 0;
   const int dmax = D > DV ? D : DV;
   if ((variant == 0 || variant == 2) && H <= 256 && dmax <= 128) {
@@ -603,7 +658,7 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
   }
   if ((variant == 3 || variant == 4) && H <= 256 && dmax <= 128) {
     int rc = 1;
-    TA_BY_WIDTH(launch_split, rc)
+    TA_BY_WIDTH(launch_split, rc, splits, (float*)scratch)
     if (rc == 0) return 0;
   }
   if (variant == 2 || variant == 4) return 2;

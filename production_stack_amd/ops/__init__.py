@@ -540,8 +540,8 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
                    token_seq: torch.Tensor, token_pos: torch.Tensor,
                    scale: float, heads: int, chunk: int = 0, window: int = 0,
                    sink: bool = False, talk: torch.Tensor = None,
-                   out: torch.Tensor = None, variant: int = 0
-                   ) -> torch.Tensor:
+                   out: torch.Tensor = None, variant: int = 0,
+                   splits: int = 0) -> torch.Tensor:
     """Paged attention of a ragged batch. q [T, H*D] (row-strided view
     allowed); token_seq/token_pos int32 [T] give each token's block-table
     row and position; talk: optional fp32 [H, H] score mix; chunk/window:
@@ -574,12 +574,25 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     assert block_tables.is_contiguous()
     if talk is not None:
         assert talk.is_contiguous()
+    # single tokens: when the batch is too small to fill the chip with one
+    # workgroup per token, each token's keys are shared out over several
+    # workgroups whose partial softmax records are merged afterwards
+    scratch = None
+    if variant not in (3, 4):
+        splits = 1
+    elif splits <= 0:
+        splits = max(1, min(8, 512 // T)) if T < 256 else 1
+    if splits > 1:
+        if True:
+            scratch = torch.empty((T, splits, H, DV + 2),
+                                  dtype=torch.float32, device=q.device)
     rc = _mx().mx_talk_attention(
         _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
         _p(v_cache), _p(block_tables), block_tables.shape[1],
         _p(token_seq), _p(token_pos), _p(talk), T, H, G, D, DV, BS,
         _f(scale), int(chunk), int(window), int(bool(sink)),
-        _mx_dtype(q.dtype), int(variant), _stream())
+        _mx_dtype(q.dtype), int(variant), int(splits), _p(scratch),
+        _stream())
     if rc != 0:
         raise RuntimeError(
             f"talk_attention: heads x dim {H}x{D}/{DV} exceeds the kernel's "

@@ -105,7 +105,7 @@ def test_kv_append_distinct_widths(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("variant", [1, 2, 4])
+@pytest.mark.parametrize("variant", [1, 2, 4, 41, 43])
 @pytest.mark.parametrize("H,G,D,DV,chunk,window,sink,talk", [
     (4, 2, 40, 40, 24, 0, True, True),
     (6, 3, 40, 24, 40, 0, True, True),
@@ -148,7 +148,9 @@ def test_talk_attention(dtype, variant, H, G, D, DV, chunk, window, sink,
     got = ops.talk_attention(
         q.cuda()[:, :H * D], kc.cuda(), vc.cuda(), tables.cuda(), ts.cuda(),
         tp.cuda(), scale, H, chunk=chunk, window=window, sink=sink,
-        talk=tk.cuda() if tk is not None else None, variant=variant)
+        talk=tk.cuda() if tk is not None else None,
+        # 41 / 43: the split-key kernel with one / three workgroups a token
+        variant=min(variant, 4), splits=variant - 40 if variant > 4 else 0)
     torch.testing.assert_close(got.cpu().float().view(T, H, DV), want,
                                **tol(dtype))
 
