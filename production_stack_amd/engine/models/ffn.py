@@ -136,6 +136,35 @@ class SparseMoE(nn.Module):
             return []
         return [self.shared.gate_up, self.shared_gate]
 
+    # decode-sized batches touch (nearly) every expert's weights anyway:
+    # up to this many rows all experts run over all rows as three batched
+    # GEMMs with the routing weight (0 for experts a row did not choose)
+    # folded in, instead of a host-side loop that needs the per-expert row
+    # counts on the host every layer
+    DENSE_MAX_ROWS = 128
+
+    def _all_experts(self, x: torch.Tensor, weights: torch.Tensor,
+                     sel: torch.Tensor) -> torch.Tensor:
+        """Every expert over every row; exact because the experts have no
+        biases: a zero-weighted input (or output) contributes exactly 0."""
+        sp = self.spec
+        T, E, ff = x.shape[0], sp.experts, sp.ff
+        wm = torch.zeros((T, E), dtype=torch.float32, device=x.device)
+        wm.scatter_(1, sel, weights)
+        wm = wm.t().unsqueeze(-1)                       # [E, T, 1]
+        if sp.weight_on_input:
+            xe = (x.float().unsqueeze(0) * wm).to(x.dtype)
+        else:
+            xe = x.unsqueeze(0).expand(E, T, x.shape[1])
+        gu = torch.bmm(xe, self.experts_gate_up.transpose(1, 2))
+        gu2 = gu.view(E * T, 2 * ff)
+        act = ops.gated_act(gu2[:, :ff], gu2[:, ff:], sp.act, sp.limit)
+        y = torch.bmm(act.view(E, T, ff), self.experts_down.transpose(1, 2))
+        y = y.float()
+        if not sp.weight_on_input:
+            y = y * wm
+        return y.sum(dim=0)
+
     def _expert(self, e: int, xe: torch.Tensor) -> torch.Tensor:
         ff = self.spec.ff
         gu = gemm_policy.linear(xe, self.experts_gate_up[e])
@@ -152,9 +181,13 @@ class SparseMoE(nn.Module):
         sp = self.spec
         weights, sel = route(x, self.router, sp.top, sp.score,
                              sp.renormalize)
-        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
-        sparse_moe(x, weights, sel, sp.experts, self._expert,
-                   weight_on_input=sp.weight_on_input, out=out)
+        T = x.shape[0]
+        if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
+            out = self._all_experts(x, weights, sel)
+        else:
+            out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            sparse_moe(x, weights, sel, sp.experts, self._expert,
+                       weight_on_input=sp.weight_on_input, out=out)
         if self.shared is not None:
             sff = sp.shared_ff
             y = self.shared.forward_from_proj(proj[:, :2 * sff])
