@@ -165,7 +165,7 @@ PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
                      const int* __restrict__ table, int j0, int nk, int G,
                      int Dw, int BS) {
   constexpr int VEC = TaVec<T>::N;
-  constexpr int U = 4;
+  constexpr int U = 8;
   const int tid = threadIdx.x, nt = blockDim.x;
   if (Dw % VEC == 0) {
     const int vpr = Dw / VEC;

@@ -1200,7 +1200,9 @@ def main() -> None:
                     help="one or more public names for this model "
                          "(vLLM-style; first is primary, the rest alias)")
     ap.add_argument("--max-model-len", type=int, default=4096)
-    ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--dtype", default="bfloat16",
+                    help="bfloat16, or float32 for model families that run "
+                         "in it (hybrid recurrent/attention stacks)")
     ap.add_argument("--max-num-seqs", type=int, default=256)
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
@@ -1277,7 +1279,9 @@ def main() -> None:
     from production_stack_amd.engine.config import ParallelConfig
 
     cfg = EngineConfig(
-        model=args.model,
+        model=args.model,  # architecture name or checkpoint folder
+        dtype=("float32" if args.dtype in ("float32", "fp32")
+               else "bfloat16"),
         max_model_len=args.max_model_len,
         seed=args.seed,
         weights_path=args.weights_path,
