@@ -164,13 +164,19 @@ def _compare_one(model: str, args, use_cuda: bool) -> dict:
                 for _ in range(n)]
 
     one = SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True)
-    engine.generate(prompts(1, min(L, 512)), one)       # warm-up
+    # untimed pass of the same shapes (GEMM heuristics, allocator, lazy
+    # kernel loading happen here, not inside the timed region)
+    engine.generate(prompts(P, L), one)
     sync()
     t0 = time.perf_counter()
     engine.generate(prompts(P, L), one)
     sync()
     prefill = P * L / (time.perf_counter() - t0)
 
+    # untimed decode steps at the timed batch size
+    engine.generate(prompts(B, 16), SamplingParams(
+        max_tokens=4, temperature=0.0, ignore_eos=True))
+    sync()
     many = SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True)
     for i, pr in enumerate(prompts(B, ctx)):
         engine.add_request(f"d{i}", pr, many)
