@@ -159,8 +159,12 @@ class LLMEngine:
                     continue
                 seq = self.scheduler.get(rid)
                 if seq is None:
+                    # prompt_logprobs set: logits are wanted at prompt
+                    # positions, so no position may be skipped through a
+                    # prefix-cache hit (the block manager honours this)
                     seq = Sequence(rid, tokens, SamplingParams(
-                        max_tokens=1, temperature=0.0, ignore_eos=True))
+                        max_tokens=1, temperature=0.0, ignore_eos=True,
+                        prompt_logprobs=0))
                     self.scheduler.add(seq)
                     self.stats.num_requests += 1
                 else:

@@ -267,3 +267,64 @@ def test_other_layer_orders_and_sizes(tmp_path, device):
     eng = make_engine(path, "float32", device)
     assert rel_err(replay(eng, "a", toks, [None]), want) < 2e-4
     assert rel_err(replay(eng, "b", toks, [5, 2, 60, 1, None]), want) < 2e-4
+
+
+ODD_STACKS = [
+    # head widths that are no multiple of 8 or 16, five query heads on one
+    # kv head, a chunk of 7 positions, every expert chosen, delta heads of
+    # 20 and 100 channels
+    ([(attn(5, 1, 20, 12, 7, 0.22), moe(12, 1.5, 3, 3, (20, 2.0))),
+      (delta(2, 20), dense(36)),
+      (delta(1, 100), None),
+      (attn(7, 7, 12, 20, 50, 0.3), dense(28))], 60, 71),
+    # one layer only; a single head everywhere
+    ([(delta(1, 16), moe(8, 3.0, 2, 1, None))], 24, 19),
+    ([(attn(1, 1, 16, 16, 5, 0.25), None)], 16, 23),
+]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("which", range(len(ODD_STACKS)))
+def test_odd_shapes(tmp_path, device, which):
+    stack, width, vocab = ODD_STACKS[which]
+    cfg = make_cfg(stack, width=width, vocab=vocab, eps=1e-6, scale=3.0)
+    W = make_weights(cfg, seed=40 + which, rank=5)
+    path = save_checkpoint(tmp_path / f"odd{which}", cfg, W)
+    toks = tokens(64, 70 + which, vocab=vocab)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, "float32", device)
+    assert rel_err(replay(eng, "a", toks, [None]), want) < 2e-4
+    assert rel_err(replay(eng, "b", toks, [6, 1, 2, 30, 1, 1, None]),
+                   want) < 2e-4
+    # two requests side by side, cut differently
+    half = replay_two(eng, toks, [9, 40, None], [33, 2, None])
+    assert rel_err(half[0], want) < 2e-4 and rel_err(half[1], want) < 2e-4
+
+
+def replay_two(eng, toks, sizes_a, sizes_b):
+    """The same tokens as two requests in shared steps with different
+    cuts; returns both requests' logits at every position."""
+    def cuts(sizes):
+        out, at = [], 0
+        for s in sizes:
+            s = len(toks) - at if s is None else min(s, len(toks) - at)
+            if s > 0:
+                out.append((at, at + s))
+                at += s
+        return out
+    ca, cb = cuts(sizes_a), cuts(sizes_b)
+    got = {"x": [], "y": []}
+    for step in range(max(len(ca), len(cb))):
+        entries, end = [], []
+        for rid, cc in (("x", ca), ("y", cb)):
+            if step < len(cc):
+                a, b = cc[step]
+                entries.append((rid, toks[a:b], list(range(b - a))))
+                if b == len(toks):
+                    end.append(rid)
+        out = eng.replay_step(entries, end=end)
+        r0 = 0
+        for rid, t, _ in entries:
+            got[rid].append(out[r0:r0 + len(t)])
+            r0 += len(t)
+    return torch.cat(got["x"]), torch.cat(got["y"])
