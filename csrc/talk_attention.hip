@@ -414,6 +414,7 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   float* sS = sV + TK * G * PITCH;   // [TK][H] raw scores
   float* sT = sS + TK * H;           // [H*H]
   float* sML = sT + H * H;           // [2][H*NS] partial max / denominator
+  float* sQ = sML + 2 * H * NS;      // [H][PITCH] query rows (fp32)
   // the merge buffer [H][DP] reuses sK after the key loop
 
   const int tid = threadIdx.x;
@@ -437,14 +438,16 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
 
   if (talk != nullptr)
     for (int c = tid; c < H * H; c += blockDim.x) sT[c] = talk[c];
-  float qv[DP], acc[DP];
-#pragma unroll
-  for (int d = 0; d < DP; ++d) {
-    qv[d] = (valid && d < D)
-                ? MxElem<T>::ld(q + (size_t)t * ldq + h * D + d)
-                : 0.f;
-    acc[d] = 0.f;
+  // the query stays in LDS (each thread scores only KPT keys a tile), so
+  // the registers hold just the output accumulator
+  for (int c = tid; c < H * DP; c += blockDim.x) {
+    const int hh = c / DP, d = c % DP;
+    sQ[hh * PITCH + d] =
+        d < D ? MxElem<T>::ld(q + (size_t)t * ldq + hh * D + d) : 0.f;
   }
+  float acc[DP];
+#pragma unroll
+  for (int d = 0; d < DP; ++d) acc[d] = 0.f;
   const bool own_sink = sink && i == 0 && ks == 0;
   float m = own_sink ? 0.f : PS_NEG_INF;
   float l = own_sink ? 1.f : 0.f;
@@ -460,14 +463,15 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
         const int jj = c * NS + i;
         if (jj < nk) {
           const float4* kr = (const float4*)(sK + (jj * G + gk) * PITCH);
+          const float4* qr = (const float4*)(sQ + h * PITCH);
           float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
           for (int d4 = 0; d4 < DP / 4; ++d4) {
-            const float4 kk = kr[d4];
-            a0 += qv[4 * d4 + 0] * kk.x;
-            a1 += qv[4 * d4 + 1] * kk.y;
-            a2 += qv[4 * d4 + 2] * kk.z;
-            a3 += qv[4 * d4 + 3] * kk.w;
+            const float4 kk = kr[d4], qq = qr[d4];
+            a0 += qq.x * kk.x;
+            a1 += qq.y * kk.y;
+            a2 += qq.z * kk.z;
+            a3 += qq.w * kk.w;
           }
           sS[jj * H + h] = ((a0 + a1) + (a2 + a3)) * scale;
         }
@@ -592,7 +596,8 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
   size_t lds = 0;
   // most slices first (threads), then most keys per tile (fewer barriers)
   for (int ns = 256 / H; ns >= 1 && KPT == 0; ns >>= 1) {
-    const size_t fixed = (size_t)H * H + 2 * H * ns;
+    const size_t fixed =
+        (size_t)H * H + 2 * H * ns + (size_t)H * (DP + 4);  // + query rows
     for (int k = 8; k >= 1; k >>= 1) {
       const size_t tk = (size_t)ns * k;
       size_t tile = 2 * tk * G * (DP + 4);
