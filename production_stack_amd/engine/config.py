@@ -422,9 +422,9 @@ def _nanurax_stack(
 ARCHITECTURES.update({
     # CPU-runnable test config
     "tiny-nanurax": _nanurax_stack(
-        "tiny-nanurax", 64, 512, 4, delta_heads=2, delta_dim=16,
-        decay_rank=8, attn_heads=4, attn_kv=2, attn_dim=16, chunk=32,
-        ff=128, experts=4, top=2, expert_ff=32, shared_ff=64),
+        "tiny-nanurax", 96, 384, 4, delta_heads=3, delta_dim=32,
+        decay_rank=8, attn_heads=6, attn_kv=3, attn_dim=16, chunk=40,
+        ff=160, experts=5, top=2, expert_ff=32, shared_ff=64),
     # llama-3.2-1b-sized stack (same width, depth, dense ff and vocab)
     "nanurax-1b": _nanurax_stack(
         "nanurax-1b", 2048, 128256, 16, delta_heads=32, delta_dim=64,
