@@ -209,9 +209,11 @@ def paged_attn_prefill_mfma(
 
 def greedy_sample(logits: torch.Tensor) -> torch.Tensor:
     if logits.is_cuda:
-        _require_ext()
-        if logits.dtype != torch.bfloat16:  # penalty-adjusted fp32 rows
+        # fp32 rows (penalty-adjusted, or families that emit fp32 logits)
+        # need no extension kernel
+        if logits.dtype != torch.bfloat16:
             return logits.float().argmax(dim=-1)
+        _require_ext()
         out = torch.empty(
             logits.shape[0], dtype=torch.long, device=logits.device
         )
