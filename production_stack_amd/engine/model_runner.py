@@ -191,6 +191,29 @@ class ModelRunner:
     def capture_decode_graphs(self, max_batch: int) -> None:
         """hipGraph-capture decode-only steps (see graph_runner.py)."""
         if (
+            self.device.type == "cuda"
+            and not self.config.enforce_eager
+            and hasattr(self.model, "gemm_weights")
+            and ops.HAVE_EXT
+            and self.model.dtype == torch.bfloat16
+        ):
+            # eager families still get the per-shape GEMM choice for
+            # decode-sized batches (hipBLASLt vs the in-house skinny /
+            # 8-phase kernels), keyed on the exact row count
+            from production_stack_amd.engine.graph_runner import BUCKETS
+            from production_stack_amd.ops import gemm_policy
+
+            try:
+                gemm_policy.tune(
+                    self.model.gemm_weights(),
+                    [b for b in BUCKETS if b <= min(max_batch, 128)],
+                    self.device)
+            except Exception:
+                import logging
+
+                logging.getLogger("engine.runner").exception(
+                    "gemm autotune failed; using hipBLASLt everywhere")
+        if (
             self.device.type != "cuda"
             or self.config.enforce_eager
             or self.pp_size > 1

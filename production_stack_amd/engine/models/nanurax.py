@@ -239,6 +239,25 @@ class NanuraxForCausalLM(nn.Module):
                    for kind, h, d, dv in self.cache_shapes()
                    if kind == "state")
 
+    def gemm_weights(self):
+        """One weight per distinct projection shape of the stack (for the
+        per-shape GEMM choice at decode batch sizes)."""
+        seen, out = set(), []
+        for layer in self.layers:
+            if layer.w_in is None:
+                layer.fuse()
+            cands = [layer.w_in, layer.w_out, layer.mixer.out_weight]
+            if hasattr(layer.mixer, "w2"):
+                cands.append(layer.mixer.w2)
+            if isinstance(layer.mlp, SparseMoE) and layer.mlp.shared:
+                cands.append(layer.mlp.shared.down)
+            for w in cands:
+                if w is not None and w.dim() == 2 and w.is_contiguous() \
+                        and tuple(w.shape) not in seen:
+                    seen.add(tuple(w.shape))
+                    out.append(w)
+        return out
+
     # ---- weights -------------------------------------------------------
     @torch.no_grad()
     def random_init(self, seed: int = 0) -> None:
