@@ -28,6 +28,8 @@
 // sizes of 16-64 seqs, seqs*kv_heads workgroups cannot fill 256 CUs and the
 // kernel runs at <10% of HBM bandwidth (measured, profiles/ run1).
 // ---------------------------------------------------------------------------
+typedef __bf16 ps_bf16pair __attribute__((ext_vector_type(2)));
+
 template <int HEAD_DIM, int GQ, int BLOCK_SIZE, int NWAVES, int LOWREG,
           typename KVT>
 // LOWREG: cap registers so 3 workgroups co-reside per SIMD (168-VGPR
@@ -124,20 +126,47 @@ __global__ __launch_bounds__(NWAVES * 64, LOWREG ? 3 : 1) void paged_attn_decode
       kvec8 kv = *(const kvec8*)(kb + tok * D + sl * 8);
       if constexpr (!LOWREG)
         vv[tt] = *(const kvec8*)(vb + tok * D + sl * 8);
-      float kf[8];
-      KVTr::to_f32x8(kv, kf);  // packed v_cvt_pk_f32_fp8 on fp8 caches
+      if constexpr (LOWREG && sizeof(KVT) == 2) {
+        // q and k are both packed bf16 pairs: one v_dot2_f32_bf16 does two
+        // multiply-adds (products exact, fp32 accumulation) with no
+        // conversion of either operand
+        union {
+          kvec8 v;
+          unsigned int u[4];
+        } kk;
+        kk.v = kv;
 #pragma unroll
-      for (int g = 0; g < GQ; g++) {
-        float s = 0.f;
+        for (int g = 0; g < GQ; g++) {
+          union {
+            ps_bf16x8 v;
+            unsigned int u[4];
+          } qq;
+          qq.v = qp[g];
+          float s = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-          if constexpr (LOWREG)
-            s += ps_bf16_to_f32(qp[g][j]) * kf[j];
-          else
-            s += qf[g][j] * kf[j];
+          for (int j = 0; j < 4; j++)
+            s = __builtin_amdgcn_fdot2_f32_bf16(
+                __builtin_bit_cast(ps_bf16pair, qq.u[j]),
+                __builtin_bit_cast(ps_bf16pair, kk.u[j]), s, false);
+          s = ps_group_sum<LPG>(s) * scale;
+          sc[g][tt] = valid ? s : PS_NEG_INF;
         }
-        s = ps_group_sum<LPG>(s) * scale;
-        sc[g][tt] = valid ? s : PS_NEG_INF;
+      } else {
+        float kf[8];
+        KVTr::to_f32x8(kv, kf);  // packed v_cvt_pk_f32_fp8 on fp8 caches
+#pragma unroll
+        for (int g = 0; g < GQ; g++) {
+          float s = 0.f;
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            if constexpr (LOWREG)
+              s += ps_bf16_to_f32(qp[g][j]) * kf[j];
+            else
+              s += qf[g][j] * kf[j];
+          }
+          s = ps_group_sum<LPG>(s) * scale;
+          sc[g][tt] = valid ? s : PS_NEG_INF;
+        }
       }
     }
     if constexpr (LOWREG) {
