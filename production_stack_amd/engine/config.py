@@ -21,13 +21,27 @@ class MixerSpec:
 
     kind "attention": softmax attention over a paged KV cache. `chunk`
     restricts every query to keys of its own aligned block of positions
-    (0 = plain causal), `window` to the trailing N keys (0 = off), `sink`
-    adds a value-less key of score 0 to the softmax denominator,
-    `talking_heads` mixes the heads' scores with a learned [H, H] matrix
-    before the softmax, `rope` applies the rotary position code.
-    kind "general_delta": gated delta-rule linear recurrence with a
-    per-sequence fp32 state of heads x dim x dim; `decay_rank` is the
-    width of the low-rank decay projection.
+    (0 = plain causal), `window` to the trailing N keys (0 = off) with the
+    first `keep_first` keys of the sequence staying visible behind it,
+    `sink` adds a value-less key to the softmax denominator (score 0, or a
+    learned per-head score with `learned_sink`), `softcap` squashes scores
+    to cap * tanh(score / cap) (0 = off), `talking_heads` mixes the heads'
+    scores with a learned [H, H] matrix before the softmax, `rope` applies
+    the rotary position code, `bias` adds projection biases to q/k/v,
+    `qk_norm` RMS-normalises every query and key head with a learned
+    weight, `v_mix` blends the layer's values with those of the first
+    `v_mix` layer of the stack (learned scalar weight).
+    kind "latent_attention": keys and values of all heads are expanded from
+    one cached latent of `kv_rank` entries per token; every head has `dim`
+    position-free query/key entries and `rot_dim` rotated ones (the rotated
+    key part is shared by the heads); `rot_dims` leading entries of the
+    rotated part turn with base `rot_base`, interleaved pairs.
+    kind "general_delta" / "channel_delta": gated delta-rule linear
+    recurrences with a per-sequence fp32 state of heads x dim x vdim;
+    `decay_rank` is the width of the low-rank decay projection
+    (general_delta), `conv` the taps of the short causal convolution on
+    q/k/v and `gate_rank` the width of the low-rank output gate
+    (channel_delta).
     """
 
     kind: str
@@ -42,6 +56,18 @@ class MixerSpec:
     talking_heads: bool = False
     rope: bool = True
     decay_rank: int = 0
+    keep_first: int = 0
+    softcap: float = 0.0
+    learned_sink: bool = False
+    bias: bool = False
+    qk_norm: bool = False
+    v_mix: bool = False
+    kv_rank: int = 0
+    rot_dim: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    conv: int = 0
+    gate_rank: int = 0
 
 
 @dataclass
@@ -73,6 +99,12 @@ class LayerSpec:
     # True: mixer and feed-forward both read one norm's output and their
     # sum joins the residual; False: sequential pre-norm sublayers
     parallel: bool = False
+    # the mixer's input is blended with the previous token's (learned
+    # per-channel weight); the previous input is per-sequence state
+    token_shift: bool = False
+    # the layer hands on a learned weighted sum of the embedding output and
+    # all layer results so far instead of its own result
+    depth_average: bool = False
 
 
 @dataclass
@@ -108,11 +140,15 @@ class ModelConfig:
     # scalar head/ff fields above then hold the stack's maxima
     layer_specs: Optional[list] = None
     embedding_scale: float = 1.0
+    # RMS norms of the stack normalise this many equal consecutive parts
+    # of the vector separately
+    norm_groups: int = 1
 
     @property
     def has_recurrent_state(self) -> bool:
         return bool(self.layer_specs) and any(
-            ls.mixer.kind != "attention" for ls in self.layer_specs)
+            ls.mixer.kind not in ("attention", "latent_attention")
+            or ls.token_shift for ls in self.layer_specs)
 
     @property
     def q_size(self) -> int:

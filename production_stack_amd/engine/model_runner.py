@@ -157,19 +157,39 @@ class ModelRunner:
                     "this model family keeps its KV cache in the serving "
                     "dtype (no fp8 KV)")
             dt = self.model.dtype
-            self.kv_caches = []
-            for kind, heads, d, dv in self.model.cache_shapes():
+            slots = max(self.num_state_slots, 1)
+
+            def alloc(desc):
+                kind = desc[0]
                 if kind == "kv":
-                    self.kv_caches.append((
+                    _, heads, d, dv = desc
+                    return (
                         torch.zeros((num_blocks, heads, bs, d), dtype=dt,
                                     device=self.device),
                         torch.zeros((num_blocks, heads, bs, dv), dtype=dt,
                                     device=self.device),
-                    ))
-                else:
-                    self.kv_caches.append(torch.zeros(
-                        (max(self.num_state_slots, 1), heads, d, dv),
-                        dtype=torch.float32, device=self.device))
+                    )
+                if kind == "paged":
+                    # one paged tensor (keys that also hold the values)
+                    _, heads, d = desc
+                    return torch.zeros((num_blocks, heads, bs, d), dtype=dt,
+                                       device=self.device)
+                if kind == "state":
+                    _, heads, d, dv = desc
+                    return torch.zeros((slots, heads, d, dv),
+                                       dtype=torch.float32,
+                                       device=self.device)
+                if kind == "slots":
+                    # per-sequence state of any shape; dtype None = the
+                    # serving dtype
+                    _, shape, sdt = desc
+                    return torch.zeros((slots, *shape), dtype=sdt or dt,
+                                       device=self.device)
+                if kind == "multi":
+                    return tuple(alloc(d) for d in desc[1])
+                raise ValueError(f"unknown cache kind {kind!r}")
+
+            self.kv_caches = [alloc(d) for d in self.model.cache_shapes()]
             return
         kh = self.model.kv_heads
         kv_dt = self.config.cache.kv_cache_dtype

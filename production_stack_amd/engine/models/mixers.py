@@ -8,7 +8,12 @@ Each mixer exposes
                 pair for attention, a per-sequence fp32 state for the
                 recurrence;
   * forward_from_proj(proj, meta, cache) -> the mixer's pre-output-projection
-                activations [T, out_in], and out_weight [width, out_in].
+                activations [T, out_in], and out_weight [width, out_in];
+  * forward(h, meta, cache, shared) -> the same from the layer input, for
+                layers whose mixer does not share its input projection
+                (`shared` is a per-step dict for tensors that later layers
+                of the stack read, e.g. the first value-mixing layer's
+                values).
 """
 
 from __future__ import annotations
@@ -31,13 +36,15 @@ DELTA_DECAY_SCALE = math.exp(-0.5)
 class TalkAttention(nn.Module):
     """Grouped-query softmax attention over the paged KV cache with the
     MixerSpec's options: no rotary code, score mixing across heads,
-    aligned-chunk / trailing-window visibility, denominator sink; key and
-    value widths may differ."""
+    aligned-chunk / trailing-window visibility (with kept first keys),
+    capped scores, denominator sink (fixed or learned), projection biases,
+    per-head query/key norm, value blending with the stack's first
+    value-mixing layer; key and value widths may differ."""
 
     kind = "attention"
 
     def __init__(self, width: int, spec: MixerSpec,
-                 dtype: torch.dtype) -> None:
+                 dtype: torch.dtype, eps: float = 1e-5) -> None:
         super().__init__()
         if spec.rope:
             raise NotImplementedError(
@@ -57,9 +64,32 @@ class TalkAttention(nn.Module):
             nn.Parameter(torch.empty(H, H, dtype=torch.float32))
             if spec.talking_heads else None)
         self.scale = spec.scale or 1.0 / math.sqrt(D)
+        self.eps = eps
+        self.qkv_bias = (
+            nn.Parameter(torch.empty(self.qkv.shape[0], dtype=dtype))
+            if spec.bias else None)
+        self.q_norm = self.k_norm = None
+        if spec.qk_norm:
+            self.q_norm = nn.Parameter(torch.empty(D, dtype=torch.float32))
+            self.k_norm = nn.Parameter(torch.empty(D, dtype=torch.float32))
+        self.sink_vals = (
+            nn.Parameter(torch.empty(H, dtype=torch.float32))
+            if spec.learned_sink else None)
+        self.vmix = (
+            nn.Parameter(torch.empty((), dtype=torch.float32))
+            if spec.v_mix else None)
 
     def in_params(self):
         return [self.qkv]
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if self.qkv_bias is not None:
+            # the bias joins the fp32 accumulator of the projection
+            proj = torch.addmm(self.qkv_bias, h, self.qkv.t())
+        else:
+            proj = gemm_policy.linear(h, self.qkv)
+        return self.forward_from_proj(proj, meta, cache, out, shared)
 
     @property
     def out_in(self) -> int:
@@ -69,15 +99,25 @@ class TalkAttention(nn.Module):
         return ("kv", self.G, self.D, self.DV)
 
     def forward_from_proj(self, proj: torch.Tensor, meta, cache,
-                          out: Optional[torch.Tensor] = None
-                          ) -> torch.Tensor:
+                          out: Optional[torch.Tensor] = None,
+                          shared: Optional[dict] = None) -> torch.Tensor:
         H, G, D, DV = self.H, self.G, self.D, self.DV
         k_cache, v_cache = cache
         q = proj[:, :H * D]
         k = proj[:, H * D:H * D + G * D]
         v = proj[:, H * D + G * D:]
-        ops.kv_append(k, v, k_cache, v_cache, meta.slot_mapping)
         sp = self.spec
+        if sp.qk_norm or sp.v_mix:
+            # the first value-mixing layer of a step publishes its values;
+            # later ones blend theirs with them before caching
+            v_first = shared.get("v_first") if sp.v_mix else None
+            ops.attn_prep(q, k, v, self.q_norm, self.k_norm, self.eps,
+                          self.vmix, v_first, k_cache, v_cache,
+                          meta.slot_mapping, H)
+            if sp.v_mix and v_first is None:
+                shared["v_first"] = v
+        else:
+            ops.kv_append(k, v, k_cache, v_cache, meta.slot_mapping)
         T = proj.shape[0]
         if out is None:
             out = torch.empty((T, H * DV), dtype=proj.dtype,
@@ -93,8 +133,99 @@ class TalkAttention(nn.Module):
                     q[a:b], k_cache, v_cache, meta.block_tables,
                     meta.token_seq[a:b], meta.positions[a:b], self.scale, H,
                     chunk=sp.chunk, window=sp.window, sink=sp.sink,
-                    talk=self.talk, out=out[a:b], variant=variant)
+                    talk=self.talk, out=out[a:b], variant=variant,
+                    keep_first=sp.keep_first, softcap=sp.softcap,
+                    sink_vals=self.sink_vals)
         return out
+
+
+class LatentAttention(nn.Module):
+    """Multi-head attention whose keys and values are low-rank expansions
+    of one cached latent per token. Per head the query has `dim`
+    position-free entries and `rot_dim` rotary ones; the key's rotary part
+    is one vector shared by all heads. The per-head up-projections are
+    folded around the attention: the position-free query part is mapped
+    into the latent space (q W_uk), attention runs as single-KV-head
+    attention over cached rows [latent | rotary key part] whose values are
+    the latent itself, and the result is expanded by W_uv. Only
+    kv_rank + rot_dim numbers per token are cached."""
+
+    kind = "latent_attention"
+
+    def __init__(self, width: int, spec: MixerSpec, dtype: torch.dtype,
+                 eps: float, max_pos: int) -> None:
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.max_pos = max_pos
+        H, D, R, L = spec.heads, spec.dim, spec.rot_dim, spec.kv_rank
+        DV = spec.vdim or D
+        self.H, self.D, self.R, self.L, self.DV = H, D, R, L, DV
+        # fused rows: q (per head [dim | rot_dim]) | latent | rotary key
+        self.in_proj = nn.Parameter(
+            torch.empty(H * (D + R) + L + R, width, dtype=dtype))
+        self.latent_norm = nn.Parameter(torch.empty(L, dtype=torch.float32))
+        self.uk = nn.Parameter(torch.empty(H, D, L, dtype=dtype))
+        self.uv = nn.Parameter(torch.empty(H, DV, L, dtype=dtype))
+        self.sink_vals = (
+            nn.Parameter(torch.empty(H, dtype=torch.float32))
+            if spec.learned_sink else None)
+        self.out_weight = nn.Parameter(
+            torch.empty(width, H * DV, dtype=dtype))
+        self.scale = spec.scale or 1.0 / math.sqrt(D + R)
+        self._cos_sin = None
+
+    def in_params(self):
+        return [self.in_proj]
+
+    @property
+    def out_in(self) -> int:
+        return self.H * self.DV
+
+    def cache_shape(self):
+        return ("paged", 1, self.L + self.R)
+
+    def cos_sin(self, device) -> torch.Tensor:
+        cs = self._cos_sin
+        if cs is None or cs.device != device:
+            sp = self.spec
+            cs = ops.rope_table(self.max_pos, sp.rot_dims or self.R,
+                                sp.rot_base, device)
+            self._cos_sin = cs
+        return cs
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        H, D, R, L, DV = self.H, self.D, self.R, self.L, self.DV
+        sp = self.spec
+        T = h.shape[0]
+        proj = gemm_policy.linear(h, self.in_proj)
+        q = proj[:, :H * (D + R)]
+        dkv = proj[:, H * (D + R):]
+        # position-free query part into the latent space: [H, T, L]
+        q_lat = torch.bmm(q.view(T, H, D + R)[:, :, :D].transpose(0, 1),
+                          self.uk)
+        qf = ops.latent_prep(
+            q_lat, q, dkv, self.latent_norm, self.eps,
+            self.cos_sin(h.device), meta.positions, cache,
+            meta.slot_mapping, H, D, R, sp.rot_dims or R)
+        o_lat = torch.empty((T, H * L), dtype=h.dtype, device=h.device)
+        npt = min(getattr(meta, "num_prefill_tokens", T) or 0, T)
+        for a, b, variant in ((0, npt, 0), (npt, T, 3)):
+            if b > a:
+                ops.talk_attention(
+                    qf[a:b], cache, cache, meta.block_tables,
+                    meta.token_seq[a:b], meta.positions[a:b], self.scale, H,
+                    sink=sp.sink, out=o_lat[a:b], variant=variant,
+                    softcap=sp.softcap, sink_vals=self.sink_vals, vdim=L)
+        # expand the attended latents per head: [H, T, L] x [H, L, DV]
+        o = torch.bmm(o_lat.view(T, H, L).transpose(0, 1),
+                      self.uv.transpose(1, 2))
+        o = o.transpose(0, 1).reshape(T, H * DV)
+        if out is not None:
+            out.copy_(o)
+            return out
+        return o
 
 
 class GeneralDelta(nn.Module):
@@ -149,10 +280,80 @@ class GeneralDelta(nn.Module):
             meta.seq_rows, self.H, self.eps, DELTA_DECAY_SCALE, out=out)
 
 
+class ChannelDelta(nn.Module):
+    """Gated delta rule with one decay per head and key channel. q, k
+    (kv_heads x dim, shared by groups of heads) and v (heads x vdim) pass a
+    short causal convolution and silu; q and k become unit vectors; the
+    decay exp(-exp(A_log) softplus(.)) and the output gate come from
+    low-rank projections, the write strength from a per-head sigmoid. The
+    read-out is RMS-normalised per head and gated. Per sequence the runner
+    keeps the fp32 state heads x dim x vdim and the convolution's last
+    taps - 1 inputs."""
+
+    kind = "channel_delta"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        H, G = spec.heads, spec.kv_heads or spec.heads
+        D, DV = spec.dim, spec.vdim or spec.dim
+        if H % G:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.H, self.G, self.D, self.DV = H, G, D, DV
+        self.K = max(int(spec.conv), 1)
+        ra, rg = spec.decay_rank, spec.gate_rank
+        self.ra, self.rg = ra, rg
+        self.C = 2 * G * D + H * DV          # convolved channels q | k | v
+        # fused rows: q | k | v | write strength | decay rank | gate rank
+        self.in_proj = nn.Parameter(
+            torch.empty(self.C + H + ra + rg, width, dtype=dtype))
+        self.conv_w = nn.Parameter(
+            torch.empty(self.C, self.K, dtype=torch.float32))
+        self.a2 = nn.Parameter(torch.empty(H * D, ra, dtype=dtype))
+        self.g2 = nn.Parameter(torch.empty(H * DV, rg, dtype=dtype))
+        self.a_log = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.dt_bias = nn.Parameter(torch.empty(H * D, dtype=torch.float32))
+        self.out_norm = nn.Parameter(torch.empty(DV, dtype=torch.float32))
+        self.out_weight = nn.Parameter(
+            torch.empty(width, H * DV, dtype=dtype))
+
+    def in_params(self):
+        return [self.in_proj]
+
+    @property
+    def out_in(self) -> int:
+        return self.H * self.DV
+
+    def cache_shape(self):
+        return ("multi", [("state", self.H, self.D, self.DV),
+                          ("slots", (self.K - 1, self.C), None)])
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        H, G, D, DV, C = self.H, self.G, self.D, self.DV, self.C
+        state, conv_state = cache
+        proj = gemm_policy.linear(h, self.in_proj)
+        qkv = ops.short_conv_silu(proj[:, :C], self.conv_w, conv_state,
+                                  meta.seq_rows)
+        beta = proj[:, C:C + H]
+        zdec = gemm_policy.linear(proj[:, C + H:C + H + self.ra], self.a2)
+        zgate = gemm_policy.linear(proj[:, C + H + self.ra:], self.g2)
+        return ops.gated_delta(
+            qkv[:, :G * D], qkv[:, G * D:2 * G * D], qkv[:, 2 * G * D:],
+            beta, zdec, zgate, self.a_log, self.dt_bias, self.out_norm,
+            state, meta.seq_rows, H, G, self.eps, out=out)
+
+
 def build_mixer(width: int, spec: MixerSpec, eps: float,
-                dtype: torch.dtype) -> nn.Module:
+                dtype: torch.dtype, max_pos: int = 8192) -> nn.Module:
     if spec.kind == "attention":
-        return TalkAttention(width, spec, dtype)
+        return TalkAttention(width, spec, dtype, eps)
+    if spec.kind == "latent_attention":
+        return LatentAttention(width, spec, dtype, eps, max_pos)
     if spec.kind == "general_delta":
         return GeneralDelta(width, spec, eps, dtype)
+    if spec.kind == "channel_delta":
+        return ChannelDelta(width, spec, eps, dtype)
     raise ValueError(f"unknown mixer kind {spec.kind!r}")

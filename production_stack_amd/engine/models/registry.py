@@ -31,9 +31,16 @@ def _nanurax_cls():
     return NanuraxForCausalLM
 
 
+def _derusun_cls():
+    from production_stack_amd.engine.models.derusun import DerusunForCausalLM
+
+    return DerusunForCausalLM
+
+
 MODEL_CLASSES: Dict[str, Callable] = {
     "llama": _llama_cls,
     "nanurax": _nanurax_cls,
+    "derusun": _derusun_cls,
 }
 
 
@@ -44,12 +51,19 @@ def _nanurax_config(path: str) -> ModelConfig:
 
 
 # config.json "architecture" -> reader(path) -> ModelConfig
+def _derusun_config(path: str) -> ModelConfig:
+    from production_stack_amd.engine.models import derusun
+
+    return derusun.config_from_dir(path)
+
+
 CONFIG_READERS: Dict[str, Callable[[str], ModelConfig]] = {
     "Nanurax": _nanurax_config,
+    "Derusun": _derusun_config,
 }
 
 # families whose layers also run in float32 (the Llama path is bf16-only)
-FP32_FAMILIES = {"nanurax"}
+FP32_FAMILIES = {"nanurax", "derusun"}
 
 
 def config_from_dir(path: str) -> ModelConfig:

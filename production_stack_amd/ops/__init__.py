@@ -473,14 +473,23 @@ def _f(v: float):
 
 
 def add_rms_norm32(x32: torch.Tensor, deltas, w32: torch.Tensor, eps: float,
-                   out_dtype: torch.dtype) -> torch.Tensor:
-    """x32 += sum(deltas) (fp32, in place; up to two deltas of out_dtype),
-    returns rms_norm(x32) * w32 rounded to out_dtype."""
+                   out_dtype: torch.dtype, groups: int = 1,
+                   out32: torch.Tensor = None) -> torch.Tensor:
+    """out32 = x32 + sum(deltas) (fp32; up to two deltas of out_dtype;
+    out32 defaults to x32, i.e. in place), returns rms_norm(out32) * w32
+    rounded to out_dtype. groups > 1: every one of `groups` equal
+    consecutive parts of a row has its own root mean square."""
     if not x32.is_cuda:
-        return reference.add_rms_norm32(x32, deltas, w32, eps, out_dtype)
+        return reference.add_rms_norm32(x32, deltas, w32, eps, out_dtype,
+                                        groups, out32)
     T, W = x32.shape
     assert x32.dtype == torch.float32 and x32.is_contiguous()
     assert w32.dtype == torch.float32 and w32.numel() == W
+    assert groups >= 1 and W % groups == 0
+    if out32 is None:
+        out32 = x32
+    assert out32.dtype == torch.float32 and out32.is_contiguous()
+    assert out32.shape == x32.shape
     deltas = list(deltas)
     if len(deltas) > 2:
         raise ValueError("at most two deltas")
@@ -489,11 +498,65 @@ def add_rms_norm32(x32: torch.Tensor, deltas, w32: torch.Tensor, eps: float,
     d0 = deltas[0] if deltas else None
     d1 = deltas[1] if len(deltas) > 1 else None
     h = torch.empty((T, W), dtype=out_dtype, device=x32.device)
-    _mx().mx_add_rms_norm32(
-        _p(h), _p(x32), _p(d0), _rows(d0, "delta") if d0 is not None else 0,
+    _mx().mx_add_group_norm32(
+        _p(h), _p(out32), _p(x32), _p(d0),
+        _rows(d0, "delta") if d0 is not None else 0,
         _p(d1), _rows(d1, "delta") if d1 is not None else 0, _p(w32),
-        _f(eps), T, W, _mx_dtype(out_dtype), _stream())
+        _f(eps), int(groups), T, W, _mx_dtype(out_dtype), _stream())
     return h
+
+
+def _check_seq_rows(seq_rows: torch.Tensor) -> None:
+    assert seq_rows.dtype == torch.int32 and seq_rows.dim() == 2
+    assert seq_rows.shape[1] == 4 and seq_rows.is_contiguous()
+
+
+def group_norm_shift(x32: torch.Tensor, w32: torch.Tensor, eps: float,
+                     groups: int, out_dtype: torch.dtype,
+                     shift: torch.Tensor, state: torch.Tensor,
+                     token_seq: torch.Tensor,
+                     seq_rows: torch.Tensor) -> torch.Tensor:
+    """Grouped RMSNorm followed by the token shift h + (h_prev - h) * shift
+    (see reference.group_norm_shift). x32 fp32 [T, W]; shift fp32 [W];
+    state fp32 [slots, W] (the previous token's normed row per sequence),
+    updated; token_seq int32 [T] gives every row's segment."""
+    if not x32.is_cuda:
+        return reference.group_norm_shift(x32, w32, eps, groups, out_dtype,
+                                          shift, state, seq_rows)
+    T, W = x32.shape
+    assert x32.dtype == torch.float32 and x32.is_contiguous()
+    assert w32.dtype == torch.float32 and w32.numel() == W
+    assert shift.dtype == torch.float32 and shift.numel() == W
+    assert state.dtype == torch.float32 and state.shape[1:] == (W,)
+    assert state.is_contiguous() and W % groups == 0
+    assert token_seq.dtype == torch.int32 and token_seq.shape == (T,)
+    _check_seq_rows(seq_rows)
+    h = torch.empty((T, W), dtype=out_dtype, device=x32.device)
+    _mx().mx_group_norm_shift(
+        _p(h), _p(x32), _p(w32), _f(eps), int(groups), _p(shift), _p(state),
+        _p(token_seq), _p(seq_rows), T, W, _mx_dtype(out_dtype), _stream())
+    return h
+
+
+def depth_mix(hist: torch.Tensor, n: int, weights: torch.Tensor,
+              base: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    """hist fp32 [streams, T, W]: stores the newest stream hist[n-1] =
+    base + delta (base fp32 [T, W], may be hist[n-1] itself; delta [T, W]
+    of the serving dtype) and returns sum_{j<n} weights[j] * hist[j] as a
+    new fp32 [T, W]."""
+    if not hist.is_cuda:
+        return reference.depth_mix(hist, n, weights, base, delta)
+    _, T, W = hist.shape
+    assert hist.dtype == torch.float32 and hist.is_contiguous()
+    assert 1 <= n <= hist.shape[0]
+    assert weights.dtype == torch.float32 and weights.numel() >= n
+    assert base.dtype == torch.float32 and base.shape == (T, W)
+    assert base.is_contiguous() and delta.shape == (T, W)
+    out = torch.empty((T, W), dtype=torch.float32, device=hist.device)
+    _mx().mx_depth_mix(
+        _p(out), _p(hist), int(n), _p(weights), _p(base), _p(delta),
+        _rows(delta, "delta"), T, W, _mx_dtype(delta.dtype), _stream())
+    return out
 
 
 def gated_act(gate: torch.Tensor, up: torch.Tensor, kind: str,
@@ -543,36 +606,50 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
                    scale: float, heads: int, chunk: int = 0, window: int = 0,
                    sink: bool = False, talk: torch.Tensor = None,
                    out: torch.Tensor = None, variant: int = 0,
-                   splits: int = 0) -> torch.Tensor:
+                   splits: int = 0, keep_first: int = 0,
+                   softcap: float = 0.0, sink_vals: torch.Tensor = None,
+                   vdim: int = 0) -> torch.Tensor:
     """Paged attention of a ragged batch. q [T, H*D] (row-strided view
     allowed); token_seq/token_pos int32 [T] give each token's block-table
     row and position; talk: optional fp32 [H, H] score mix; chunk/window:
-    visibility limits (0 = off); sink: add 1 to the softmax denominator.
+    visibility limits (0 = off), the first keep_first keys of a sequence
+    stay visible behind the window; softcap > 0: scores become cap *
+    tanh(score / cap); sink: a value-less key joins the softmax
+    denominator with score 0, or sink_vals[h] (fp32 [H]) when given; vdim:
+    the values are the first vdim entries of v_cache's rows (v_cache may be
+    k_cache itself: keys that carry their values).
     variant 0 picks the kernel for prompt portions (tiled thread-per-
     (head, query) where the shape fits), 3 for single tokens (split-key),
     both falling back to the plain one-workgroup-per-token kernel; 1 / 2 /
     4 force plain / tiled / split-key.
     Returns [T, H*DV]."""
     NB, G, BS, D = k_cache.shape
-    DV = v_cache.shape[3]
+    VR = v_cache.shape[3]
+    DV = vdim or VR
     T = q.shape[0]
     H = heads
-    assert q.shape == (T, H * D) and H % G == 0
+    assert q.shape == (T, H * D) and H % G == 0 and DV <= VR
+    assert v_cache.shape[:3] == (NB, G, BS)
     assert token_seq.dtype == torch.int32 and token_pos.dtype == torch.int32
     assert token_seq.shape == (T,) and token_pos.shape == (T,)
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2
     if talk is not None:
         assert talk.dtype == torch.float32 and talk.shape == (H, H)
+    if sink_vals is not None:
+        assert sink and sink_vals.dtype == torch.float32
+        assert sink_vals.shape == (H,)
     if out is None:
         out = torch.empty((T, H * DV), dtype=q.dtype, device=q.device)
     assert out.shape == (T, H * DV) and out.dtype == q.dtype
     if not q.is_cuda:
         o = reference.talk_attention(
             q.reshape(T, H, D), k_cache, v_cache, block_tables, token_seq,
-            token_pos, scale, chunk, window, sink, talk)
+            token_pos, scale, chunk, window, sink, talk, keep_first,
+            softcap, sink_vals, DV)
         out.copy_(o.reshape(T, H * DV))
         return out
     assert q.dtype == k_cache.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert block_tables.is_contiguous()
     if talk is not None:
         assert talk.is_contiguous()
@@ -585,20 +662,173 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     elif splits <= 0:
         splits = max(1, min(8, 512 // T)) if T < 256 else 1
     if splits > 1:
-        if True:
-            scratch = torch.empty((T, splits, H, DV + 2),
-                                  dtype=torch.float32, device=q.device)
+        scratch = torch.empty((T, splits, H, DV + 2),
+                              dtype=torch.float32, device=q.device)
     rc = _mx().mx_talk_attention(
         _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
         _p(v_cache), _p(block_tables), block_tables.shape[1],
         _p(token_seq), _p(token_pos), _p(talk), T, H, G, D, DV, BS,
         _f(scale), int(chunk), int(window), int(bool(sink)),
         _mx_dtype(q.dtype), int(variant), int(splits), _p(scratch),
-        _stream())
+        int(keep_first), _f(softcap), _p(sink_vals), int(VR), _stream())
     if rc != 0:
         raise RuntimeError(
             f"talk_attention: heads x dim {H}x{D}/{DV} exceeds the kernel's "
             "LDS budget")
+    return out
+
+
+def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+              q_w, k_w, eps: float, vmix, v_first, k_cache: torch.Tensor,
+              v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+              heads: int) -> None:
+    """Per-head query/key RMSNorm (weights q_w / k_w fp32 [D], None = no
+    norm; q is rewritten in place), value blend (1 - vmix) v + vmix v_first
+    when v_first [T, G*DV] is given (vmix a 0-dim fp32 tensor; v is
+    rewritten in place), and append of the keys and values to the paged
+    caches [NB, G, BS, D|DV]. q/k/v are row-strided views."""
+    NB, G, BS, D = k_cache.shape
+    DV = v_cache.shape[3]
+    T = q.shape[0]
+    H = heads
+    assert q.shape == (T, H * D) and k.shape == (T, G * D)
+    assert v.shape == (T, G * DV) and v_cache.shape[:3] == (NB, G, BS)
+    assert slot_mapping.dtype == torch.long and slot_mapping.shape == (T,)
+    if v_first is not None:
+        assert v_first.shape == v.shape and v_first.dtype == v.dtype
+        assert vmix.dtype == torch.float32 and vmix.numel() == 1
+    if not q.is_cuda:
+        reference.attn_prep(q, k, v, q_w, k_w, eps, vmix, v_first, k_cache,
+                            v_cache, slot_mapping, H)
+        return
+    assert q.dtype == k.dtype == v.dtype == k_cache.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    for w in (q_w, k_w):
+        if w is not None:
+            assert w.dtype == torch.float32 and w.numel() == D
+    _mx().mx_attn_prep(
+        _p(q), _rows(q, "q"), _p(k), _rows(k, "k"), _p(v), _rows(v, "v"),
+        _p(q_w), _p(k_w), _f(eps), _p(vmix if v_first is not None else None),
+        _p(v_first), _rows(v_first, "v_first") if v_first is not None else 0,
+        _p(k_cache), _p(v_cache), _p(slot_mapping), T, H, G, D, DV, BS,
+        _mx_dtype(q.dtype), _stream())
+
+
+def rope_table(max_pos: int, dims: int, base: float,
+               device=None) -> torch.Tensor:
+    """fp32 [max_pos, dims/2, 2] (cos, sin) of position * base^(-2i/dims),
+    angles in fp32."""
+    return reference.rope_table(max_pos, dims, base, device)
+
+
+def latent_prep(q_lat: torch.Tensor, q: torch.Tensor, dkv: torch.Tensor,
+                norm_w: torch.Tensor, eps: float, cos_sin: torch.Tensor,
+                positions: torch.Tensor, cache: torch.Tensor,
+                slot_mapping: torch.Tensor, heads: int, dim: int,
+                rot_dim: int, rot_dims: int) -> torch.Tensor:
+    """Inputs of latent attention (see reference.latent_prep): normalises
+    the latent, turns the shared key part and the queries' rotated parts
+    by their positions, appends [latent | key part] to the paged cache
+    [NB, 1, BS, L+rot_dim] and returns the queries [T, H*(L+rot_dim)]."""
+    H = heads
+    T = q.shape[0]
+    L = dkv.shape[1] - rot_dim
+    assert q.shape == (T, H * (dim + rot_dim))
+    assert q_lat.shape == (H, T, L) and q_lat.is_contiguous()
+    assert cache.shape[1] == 1 and cache.shape[3] == L + rot_dim
+    assert rot_dims % 2 == 0 and rot_dims <= rot_dim
+    assert cos_sin.dtype == torch.float32
+    assert cos_sin.shape[1:] == (rot_dims // 2, 2)
+    assert positions.dtype == torch.int32 and positions.shape == (T,)
+    assert slot_mapping.dtype == torch.long and slot_mapping.shape == (T,)
+    if not q.is_cuda:
+        return reference.latent_prep(
+            q_lat, q, dkv, norm_w, eps, cos_sin, positions, cache,
+            slot_mapping, H, dim, rot_dim, rot_dims, q.dtype)
+    assert q.dtype == dkv.dtype == q_lat.dtype == cache.dtype
+    assert norm_w.dtype == torch.float32 and norm_w.numel() == L
+    assert cache.is_contiguous() and cos_sin.is_contiguous()
+    out = torch.empty((T, H * (L + rot_dim)), dtype=q.dtype, device=q.device)
+    _mx().mx_latent_prep(
+        _p(out), _p(q_lat), _p(q), _rows(q, "q"), _p(dkv),
+        _rows(dkv, "dkv"), _p(norm_w), _f(eps), _p(cos_sin),
+        int(cos_sin.shape[0]), int(rot_dims), _p(positions), _p(cache),
+        _p(slot_mapping), T, H, dim, rot_dim, L, cache.shape[2],
+        _mx_dtype(q.dtype), _stream())
+    return out
+
+
+def short_conv_silu(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
+                    seq_rows: torch.Tensor,
+                    out: torch.Tensor = None) -> torch.Tensor:
+    """Causal per-channel convolution over time + silu over a ragged batch
+    (see reference.short_conv_silu). x [T, C] row-strided view; w fp32
+    [C, K]; state [slots, K-1, C] of x's dtype, updated."""
+    T, C = x.shape
+    K = w.shape[1]
+    assert w.dtype == torch.float32 and w.shape == (C, K) and K >= 1
+    assert state.shape[1:] == (K - 1, C) and state.dtype == x.dtype
+    if out is None:
+        out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    assert out.shape == (T, C) and out.dtype == x.dtype
+    if not x.is_cuda:
+        out.copy_(reference.short_conv_silu(x, w, state, seq_rows, x.dtype))
+        return out
+    _check_seq_rows(seq_rows)
+    assert w.is_contiguous() and state.is_contiguous()
+    rc = _mx().mx_short_conv_silu(
+        _p(out), _rows(out, "out"), _p(x), _rows(x, "x"), _p(w), _p(state),
+        _p(seq_rows), seq_rows.shape[0], C, K, T, _mx_dtype(x.dtype),
+        _stream())
+    if rc != 0:
+        raise RuntimeError(f"short_conv_silu: {K} taps are not built (1-8)")
+    return out
+
+
+def gated_delta(q, k, v, beta, zdec, zgate, a_log, dt_bias, normw, state,
+                seq_rows, heads: int, kv_heads: int, eps: float,
+                out: torch.Tensor = None) -> torch.Tensor:
+    """Gated delta rule with per-(head, key channel) decay over a ragged
+    batch (see reference.gated_delta). q/k [T, G*D], v [T, H*DV], beta
+    [T, H], zdec [T, H*D], zgate [T, H*DV]: row-strided views of one
+    dtype; a_log fp32 [H], dt_bias fp32 [H*D], normw fp32 [DV]; state fp32
+    [slots, H, D, DV], updated in place. Returns [T, H*DV]."""
+    T = q.shape[0]
+    H, G = heads, kv_heads
+    D = q.shape[1] // G
+    DV = v.shape[1] // H
+    assert H % G == 0 and q.shape == (T, G * D) and k.shape == (T, G * D)
+    assert v.shape == (T, H * DV) and beta.shape == (T, H)
+    assert zdec.shape == (T, H * D) and zgate.shape == (T, H * DV)
+    assert state.dtype == torch.float32 and state.shape[1:] == (H, D, DV)
+    for t in (k, v, beta, zdec, zgate):
+        assert t.dtype == q.dtype
+    assert a_log.dtype == torch.float32 and a_log.numel() == H
+    assert dt_bias.dtype == torch.float32 and dt_bias.numel() == H * D
+    assert normw.dtype == torch.float32 and normw.numel() == DV
+    if out is None:
+        out = torch.empty((T, H * DV), dtype=q.dtype, device=q.device)
+    assert out.shape == (T, H * DV) and out.dtype == q.dtype
+    if not q.is_cuda:
+        y = reference.gated_delta(
+            q.reshape(T, G, D), k.reshape(T, G, D), v.reshape(T, H, DV),
+            beta, zdec.reshape(T, H, D), zgate.reshape(T, H, DV), a_log,
+            dt_bias, normw, state, seq_rows, H, G, eps, q.dtype)
+        out.copy_(y.reshape(T, H * DV))
+        return out
+    _check_seq_rows(seq_rows)
+    assert state.is_contiguous()
+    rc = _mx().mx_gated_delta(
+        _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k),
+        _rows(k, "k"), _p(v), _rows(v, "v"), _p(beta), _rows(beta, "beta"),
+        _p(zdec), _rows(zdec, "zdec"), _p(zgate), _rows(zgate, "zgate"),
+        _p(a_log), _p(dt_bias), _p(normw), _p(state), _p(seq_rows),
+        seq_rows.shape[0], H, G, D, DV, _f(eps), _f(D ** -0.5),
+        _mx_dtype(q.dtype), _stream())
+    if rc != 0:
+        raise RuntimeError(
+            f"gated_delta: state {D}x{DV} per head is not built "
+            "(dims up to 256)")
     return out
 
 

@@ -210,16 +210,54 @@ def embed_scale(tokens, embed, scale: float) -> torch.Tensor:
     return embed[tokens].float() * scale
 
 
-def add_rms_norm32(x32, deltas, w32, eps: float, out_dtype):
-    """x32 += sum(deltas) in fp32 (in place); returns norm(x32) * w32 in
-    out_dtype."""
+def add_rms_norm32(x32, deltas, w32, eps: float, out_dtype, groups: int = 1,
+                   out32=None):
+    """out32 = x32 + sum(deltas) in fp32 (out32 defaults to x32: in place);
+    returns norm(out32) * w32 in out_dtype. With groups > 1 every one of
+    `groups` equal consecutive parts of a row is divided by its own root
+    mean square."""
+    if out32 is None:
+        out32 = x32
     if deltas:
         acc = deltas[0].float()
         for d in deltas[1:]:
             acc = acc + d.float()
-        x32 += acc
-    var = x32.pow(2).mean(dim=-1, keepdim=True)
-    return (x32 * torch.rsqrt(var + eps) * w32).to(out_dtype)
+        torch.add(x32, acc, out=out32)
+    elif out32 is not x32:
+        out32.copy_(x32)
+    return (_group_unit(out32, eps, groups) * w32).to(out_dtype)
+
+
+def _group_unit(x32, eps: float, groups: int):
+    T, W = x32.shape
+    p = x32.view(T, groups, W // groups)
+    return (p * torch.rsqrt(p.pow(2).mean(-1, keepdim=True) + eps)).view(T, W)
+
+
+def group_norm_shift(x32, w32, eps: float, groups: int, out_dtype, shift,
+                     state, seq_rows):
+    """h = groupnorm(x32) * w32, then every row is blended with its
+    predecessor's h: h + (h_prev - h) * shift (fp32, one rounding). The
+    predecessor of a segment's first row is state[slot] (zeros when the
+    segment starts at position 0); state[slot] becomes the h of the
+    segment's last row. seq_rows [S, 4] = (first row, rows, first
+    position, slot)."""
+    h = _group_unit(x32, eps, groups) * w32
+    out = torch.empty_like(h)
+    for t0, n, p0, slot in seq_rows.tolist():
+        prev = torch.empty_like(h[t0:t0 + n])
+        prev[0] = state[slot] if p0 > 0 else 0.0
+        prev[1:] = h[t0:t0 + n - 1]
+        out[t0:t0 + n] = h[t0:t0 + n] + (prev - h[t0:t0 + n]) * shift
+        state[slot] = h[t0 + n - 1]
+    return out.to(out_dtype)
+
+
+def depth_mix(hist, n: int, weights, base, delta):
+    """hist fp32 [streams, T, W]. The newest stream hist[n-1] = base +
+    delta (fp32) is stored, and sum_{j<n} weights[j] * hist[j] returned."""
+    torch.add(base, delta.float(), out=hist[n - 1])
+    return torch.einsum("j,jtw->tw", weights[:n].float(), hist[:n])
 
 
 def gated_act(gate, up, kind: str, limit: float, out_dtype):
@@ -254,12 +292,17 @@ def kv_append(k, v, k_cache, v_cache, slot_mapping) -> None:
 
 def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
                    scale: float, chunk: int, window: int, sink: bool,
-                   talk):
+                   talk, keep_first: int = 0, softcap: float = 0.0,
+                   sink_vals=None, vdim: int = 0):
     """Paged attention with optional head-mixed scores, aligned-chunk or
-    trailing-window visibility and a denominator sink. q [T, H, D];
-    returns [T, H, DV] in q's dtype; all score math in fp32."""
+    trailing-window visibility (the first keep_first keys stay visible
+    behind the window), capped scores and a denominator sink (score 0, or
+    sink_vals[h]). q [T, H, D]; the values are the first vdim entries of
+    v_cache rows (all of them when 0; v_cache may be k_cache). Returns
+    [T, H, DV] in q's dtype; all score math in fp32."""
     T, H, D = q.shape
-    G, bs, DV = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    G, bs = v_cache.shape[1], v_cache.shape[2]
+    DV = vdim or v_cache.shape[3]
     rep = H // G
     out = torch.zeros(T, H, DV, dtype=torch.float32)
     tk = talk.float() if talk is not None else None
@@ -271,25 +314,166 @@ def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
         if window > 0:
             lo = max(lo, pos - window + 1)
         idx = torch.arange(lo, pos + 1)
+        if keep_first > 0 and lo > 0:
+            idx = torch.cat([torch.arange(0, min(keep_first, lo)), idx])
         table = block_tables[int(token_seq[t])].long()
         blk = table[idx // bs]
         off = idx % bs
         kk = k_cache[blk, :, off].float()          # [n, G, D]
-        vv = v_cache[blk, :, off].float()          # [n, G, DV]
+        vv = v_cache[blk, :, off][..., :DV].float()  # [n, G, DV]
         kk = kk.repeat_interleave(rep, dim=1)      # [n, H, D]
         vv = vv.repeat_interleave(rep, dim=1)
         s = torch.einsum("hd,nhd->hn", q[t].float(), kk) * scale
         if tk is not None:
             s = tk @ s
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
         m = s.max(dim=-1, keepdim=True).values
         if sink:
-            m = torch.clamp(m, min=0.0)
+            s0 = (sink_vals.float().view(H, 1) if sink_vals is not None
+                  else torch.zeros(H, 1))
+            m = torch.maximum(m, s0)
         e = torch.exp(s - m)
         den = e.sum(-1, keepdim=True)
         if sink:
-            den = den + torch.exp(-m)
+            den = den + torch.exp(s0 - m)
         out[t] = torch.einsum("hn,nhv->hv", e / den, vv)
     return out.to(q.dtype)
+
+
+def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
+              v_cache, slot_mapping, heads: int):
+    """Query/key head norm, value blend and cache append of one attention
+    layer. q [T, H*D] is normalised in place per head (x / rms(x) * q_w,
+    fp32 math); k [T, G*D] likewise with k_w and appended; v [T, G*DV]
+    becomes (1 - vmix) v + vmix v_first when v_first is given (vmix a
+    0-dim fp32 tensor), is written back, and appended. q_w / k_w None:
+    no norm."""
+    T = q.shape[0]
+    G, bs, D = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    DV = v_cache.shape[3]
+    if q_w is not None:
+        qf = q.float().view(T, heads, D)
+        qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_w
+        q.copy_(qf.view(T, heads * D).to(q.dtype))
+    kf = k.float().view(T, G, D)
+    if k_w is not None:
+        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_w
+    vf = v.float()
+    if v_first is not None:
+        lam = vmix.float()
+        vf = (1.0 - lam) * vf + lam * v_first.float()
+        v.copy_(vf.to(v.dtype))
+    kv_append(kf, vf.view(T, G, DV), k_cache, v_cache, slot_mapping)
+
+
+def rope_table(max_pos: int, dims: int, base: float, device=None):
+    """fp32 [max_pos, dims/2, 2] = (cos, sin) of position * base^(-2i/dims)."""
+    i = torch.arange(0, dims, 2, dtype=torch.float32, device=device)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float32,
+                               device=device), -i / dims)
+    a = torch.arange(max_pos, dtype=torch.float32, device=device)[:, None] * f
+    return torch.stack([torch.cos(a), torch.sin(a)], dim=-1).contiguous()
+
+
+def _rotate(x, cs, dims: int):
+    """x fp32 [..., n]; cs [..., dims/2, 2] broadcastable; interleaved
+    pairs (2i, 2i+1) of the first dims entries turn."""
+    x = x.clone()
+    u, w = x[..., 0:dims:2].clone(), x[..., 1:dims:2].clone()
+    c, s = cs[..., 0], cs[..., 1]
+    x[..., 0:dims:2] = u * c - w * s
+    x[..., 1:dims:2] = w * c + u * s
+    return x
+
+
+def latent_prep(q_lat, q, dkv, norm_w, eps: float, cos_sin, positions,
+                cache, slot_mapping, heads: int, dim: int, rot_dim: int,
+                rot_dims: int, out_dtype):
+    """Inputs of latent attention for one step. q_lat [H, T, L]: the
+    position-free query parts already mapped into the latent space; q
+    [T, H*(dim+rot_dim)]: its rotated parts are taken and turned; dkv
+    [T, L+rot_dim]: the first L entries are RMS-normalised (norm_w) into
+    the latent, the rest is the shared rotated key part. The cache
+    [NB, 1, BS, L+rot_dim] receives [latent | turned key part]; returns
+    the queries [T, H*(L+rot_dim)] = per head [q_lat | turned part]."""
+    H = heads
+    T = q.shape[0]
+    L = dkv.shape[1] - rot_dim
+    cs = cos_sin[positions.long()]                        # [T, dims/2, 2]
+    c = dkv[:, :L].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+    kr = _rotate(dkv[:, L:].float(), cs, rot_dims)
+    row = torch.cat([c, kr], dim=-1)
+    bs = cache.shape[2]
+    cache[(slot_mapping // bs).long(), 0, (slot_mapping % bs).long()] = \
+        row.to(cache.dtype)
+    qr = q.float().view(T, H, dim + rot_dim)[..., dim:]
+    qr = _rotate(qr, cs[:, None], rot_dims)
+    full = torch.cat([q_lat.float().transpose(0, 1), qr], dim=-1)
+    return full.reshape(T, H * (L + rot_dim)).to(out_dtype)
+
+
+def short_conv_silu(x, w, state, seq_rows, out_dtype):
+    """Causal per-channel convolution over time followed by silu. x [T, C];
+    w fp32 [C, K] (last column weighs the current token); state
+    [slots, K-1, C] holds a sequence's last K-1 inputs (oldest first) and is
+    updated; a segment at position 0 starts from zeros."""
+    T, C = x.shape
+    K = w.shape[1]
+    y = torch.empty(T, C, dtype=torch.float32)
+    for t0, n, p0, slot in seq_rows.tolist():
+        past = state[slot].float() if p0 > 0 else torch.zeros(K - 1, C)
+        ext = torch.cat([past, x[t0:t0 + n].float()], dim=0)   # [K-1+n, C]
+        acc = torch.zeros(n, C)
+        for j in range(K):
+            acc += ext[j:j + n] * w[:, j]
+        y[t0:t0 + n] = acc
+        if K > 1:
+            state[slot] = ext[n:].to(state.dtype)
+    return (y * torch.sigmoid(y)).to(out_dtype)
+
+
+def gated_delta(q, k, v, beta, zdec, zgate, a_log, dt_bias, normw, state,
+                seq_rows, heads: int, kv_heads: int, eps: float, out_dtype):
+    """Gated delta rule with a per-(head, key channel) decay over a ragged
+    batch. q/k [T, G, D], v [T, H, DV], beta [T, H] (pre-sigmoid), zdec
+    [T, H, D] (pre-softplus, without dt_bias), zgate [T, H, DV]
+    (pre-sigmoid); a_log fp32 [H], dt_bias fp32 [H*D], normw fp32 [DV];
+    state fp32 [slots, H, D, DV] updated in place. Per token and head
+      q, k <- unit vectors (q also times D^-1/2),
+      g = exp(-exp(a_log) * softplus(zdec + dt_bias)),
+      S <- diag(g) S;  u = sigmoid(beta) (v - S^T k);  S <- S + k u^T;
+      o = S^T q,
+    then o / rms(o) * normw * sigmoid(zgate)."""
+    T, G, D = q.shape
+    H = heads
+    DV = v.shape[2]
+    rep = H // G
+    qf = q.float()
+    kf = k.float()
+    qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+    kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qf = qf.repeat_interleave(rep, dim=1)
+    kf = kf.repeat_interleave(rep, dim=1)
+    g = torch.exp(-torch.exp(a_log.float()).view(1, H, 1)
+                  * torch.nn.functional.softplus(
+                      zdec.float() + dt_bias.view(1, H, D)))
+    b = torch.sigmoid(beta.float())
+    out = torch.empty(T, H, DV, dtype=torch.float32)
+    for t0, n, p0, slot in seq_rows.tolist():
+        S = state[slot]
+        if p0 == 0:
+            S.zero_()
+        for t in range(t0, t0 + n):
+            S.mul_(g[t].unsqueeze(-1))
+            sk = torch.einsum("hi,hij->hj", kf[t], S)
+            u = b[t].unsqueeze(-1) * (v[t].float() - sk)
+            S.add_(kf[t].unsqueeze(-1) * u.unsqueeze(1))
+            out[t] = torch.einsum("hij,hi->hj", S, qf[t])
+    y = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+    y = y * normw.view(1, 1, DV) * torch.sigmoid(zgate.float())
+    return y.to(out_dtype)
 
 
 def delta_rule(r, k, v, zw, za, g, w0, ab, normw, state, seq_rows,
