@@ -1,0 +1,265 @@
+// Per-token preparation kernels of the attention and recurrent mixers:
+//   attn_prep        per-head query/key RMSNorm, value blend with another
+//                    layer's values, paged K/V append;
+//   latent_prep      latent RMSNorm, rotary turn of the shared key part and
+//                    of the queries' rotary parts, paged append of
+//                    [latent | key part], assembly of the latent-space
+//                    queries;
+//   short_conv_silu  causal per-channel convolution over time + silu with
+//                    the last taps-1 inputs of every sequence as state.
+// All arithmetic is fp32; the element type decides loads and the final
+// rounding.
+#include "mix_common.h"
+
+// One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prep_kernel(
+    T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
+    T* __restrict__ v, int ldv, const float* __restrict__ qw,
+    const float* __restrict__ kw, float eps, const float* __restrict__ vmix,
+    const T* __restrict__ vfirst, int ldvf, T* __restrict__ kc,
+    T* __restrict__ vc, const int64_t* __restrict__ slots, int H, int G,
+    int D, int DV, int BS) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int64_t slot = slots[t];
+  const int64_t blk = slot >= 0 ? slot / BS : 0;
+  const int off = slot >= 0 ? (int)(slot % BS) : 0;
+  for (int hh = wave; hh < H + G; hh += nw) {
+    const bool is_q = hh < H;
+    const int g = hh - H;
+    const T* src = is_q ? q + (size_t)t * ldq + hh * D
+                        : k + (size_t)t * ldk + g * D;
+    const float* wgt = is_q ? qw : kw;
+    float inv = 1.f;
+    if (wgt != nullptr) {
+      float ss = 0.f;
+      for (int d = lane; d < D; d += 64) {
+        const float x = MxElem<T>::ld(src + d);
+        ss += x * x;
+      }
+      ss = mx_wave_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    if (is_q) {
+      if (wgt != nullptr) {
+        T* dst = q + (size_t)t * ldq + hh * D;
+        for (int d = lane; d < D; d += 64)
+          MxElem<T>::st(dst + d, MxElem<T>::ld(src + d) * inv * wgt[d]);
+      }
+    } else if (slot >= 0) {
+      T* dst = kc + ((blk * G + g) * BS + off) * (int64_t)D;
+      for (int d = lane; d < D; d += 64) {
+        const float x = MxElem<T>::ld(src + d);
+        MxElem<T>::st(dst + d, wgt != nullptr ? x * inv * wgt[d] : x);
+      }
+    }
+  }
+  const float lam = vfirst != nullptr ? vmix[0] : 0.f;
+  for (int c = threadIdx.x; c < G * DV; c += blockDim.x) {
+    float x = MxElem<T>::ld(v + (size_t)t * ldv + c);
+    if (vfirst != nullptr) {
+      x = (1.0f - lam) * x + lam * MxElem<T>::ld(vfirst + (size_t)t * ldvf + c);
+      MxElem<T>::st(v + (size_t)t * ldv + c, x);
+    }
+    if (slot >= 0) {
+      const int g = c / DV, d = c % DV;
+      MxElem<T>::st(vc + ((blk * G + g) * BS + off) * (int64_t)DV + d, x);
+    }
+  }
+}
+
+// Turn the pair (u, w) by the table entry (cos, sin).
+PS_DEV void mx_turn(float u, float w, const float* cs, float* ou, float* ow) {
+  *ou = u * cs[0] - w * cs[1];
+  *ow = w * cs[0] + u * cs[1];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(
+    T* __restrict__ qf, const T* __restrict__ qlat, const T* __restrict__ q,
+    int ldq, const T* __restrict__ dkv, int lddkv,
+    const float* __restrict__ normw, float eps,
+    const float* __restrict__ cos_sin, int table_rows, int rot_dims,
+    const int* __restrict__ positions, T* __restrict__ cache,
+    const int64_t* __restrict__ slots, int T_, int H, int D, int R, int L,
+    int BS) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const int pos = min(max(positions[t], 0), table_rows - 1);
+  const float* cs = cos_sin + (size_t)pos * rot_dims;  // [rot_dims/2][2]
+  const T* row = dkv + (size_t)t * lddkv;
+  const int64_t slot = slots[t];
+  T* crow = cache + (slot >= 0 ? slot : 0) * (int64_t)(L + R);
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < L; c += blockDim.x) {
+    const float x = MxElem<T>::ld(row + c);
+    ss += x * x;
+  }
+  ss = mx_block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)L + eps);
+  if (slot >= 0) {
+    for (int c = threadIdx.x; c < L; c += blockDim.x)
+      MxElem<T>::st(crow + c, MxElem<T>::ld(row + c) * inv * normw[c]);
+    // shared key part: pairs below rot_dims turn, the rest passes
+    for (int i = threadIdx.x; i < R / 2; i += blockDim.x) {
+      float u = MxElem<T>::ld(row + L + 2 * i);
+      float w = MxElem<T>::ld(row + L + 2 * i + 1);
+      if (2 * i < rot_dims) mx_turn(u, w, cs + 2 * i, &u, &w);
+      MxElem<T>::st(crow + L + 2 * i, u);
+      MxElem<T>::st(crow + L + 2 * i + 1, w);
+    }
+    if ((R & 1) && threadIdx.x == 0)
+      crow[L + R - 1] = row[L + R - 1];
+  }
+  // queries: per head [latent-space part | turned rotary part]
+  const int QW = L + R;
+  for (int c = threadIdx.x; c < H * L; c += blockDim.x) {
+    const int h = c / L, l = c - h * L;
+    qf[(size_t)t * H * QW + h * QW + l] = qlat[((size_t)h * T_ + t) * L + l];
+  }
+  for (int c = threadIdx.x; c < H * (R / 2); c += blockDim.x) {
+    const int h = c / (R / 2), i = c - h * (R / 2);
+    const T* src = q + (size_t)t * ldq + h * (D + R) + D;
+    float u = MxElem<T>::ld(src + 2 * i);
+    float w = MxElem<T>::ld(src + 2 * i + 1);
+    if (2 * i < rot_dims) mx_turn(u, w, cs + 2 * i, &u, &w);
+    T* dst = qf + (size_t)t * H * QW + h * QW + L;
+    MxElem<T>::st(dst + 2 * i, u);
+    MxElem<T>::st(dst + 2 * i + 1, w);
+  }
+  if (R & 1)
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
+      qf[(size_t)t * H * QW + h * QW + QW - 1] =
+          q[(size_t)t * ldq + h * (D + R) + D + R - 1];
+}
+
+// Thread = channel, workgroup = (channel tile, segment, chunk of CONV_CH
+// tokens). A thread keeps the K-1 inputs before its current token in
+// registers. Only chunk 0 of a segment reads the sequence's state, and it
+// writes the new state (the segment's last K-1 inputs) afterwards, so no
+// other workgroup races with it.
+#define CONV_CH 64
+
+template <typename T, int K>
+__global__ __launch_bounds__(256) void short_conv_silu_kernel(
+    T* __restrict__ y, int ldy, const T* __restrict__ x, int ldx,
+    const float* __restrict__ w, T* __restrict__ state,
+    const int* __restrict__ seq_rows, int C) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int* sr = seq_rows + 4 * blockIdx.y;
+  const int t0 = sr[0], n = sr[1], p0 = sr[2], slot = sr[3];
+  const int a = blockIdx.z * CONV_CH;
+  if (c >= C || a >= n) return;
+  const int b = min(n, a + CONV_CH);
+  constexpr int P = K > 1 ? K - 1 : 1;
+  float wk[K], win[P], old[P];
+#pragma unroll
+  for (int j = 0; j < K; ++j) wk[j] = w[(size_t)c * K + j];
+  T* st = state + (size_t)slot * (K - 1) * C;
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) {
+    const int r = a - (K - 1) + j;  // row of the segment, < 0: before it
+    if (r >= 0)
+      win[j] = MxElem<T>::ld(x + (size_t)(t0 + r) * ldx + c);
+    else
+      win[j] = p0 > 0 ? MxElem<T>::ld(st + (size_t)(K - 1 + r) * C + c) : 0.f;
+    old[j] = win[j];
+  }
+  for (int t = a; t < b; ++t) {
+    const float cur = MxElem<T>::ld(x + (size_t)(t0 + t) * ldx + c);
+    float acc = wk[K - 1] * cur;
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) acc += wk[j] * win[j];
+#pragma unroll
+    for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
+    if (K > 1) win[K - 2] = cur;
+    MxElem<T>::st(y + (size_t)(t0 + t) * ldy + c, acc * mx_sigmoid(acc));
+  }
+  if (a == 0) {
+    // old[] holds the previous state (a == 0: rows -(K-1) .. -1)
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      const int r = n - (K - 1) + j;
+      float val;
+      if (r >= 0) {
+        val = MxElem<T>::ld(x + (size_t)(t0 + r) * ldx + c);
+      } else {
+        val = 0.f;
+#pragma unroll
+        for (int e = 0; e < K - 1; ++e)
+          if (e == K - 1 + r) val = old[e];
+      }
+      MxElem<T>::st(st + (size_t)j * C + c, val);
+    }
+  }
+}
+
+extern "C" {
+
+void mx_attn_prep(void* q, int ldq, const void* k, int ldk, void* v, int ldv,
+                  const void* qw, const void* kw, float eps, const void* vmix,
+                  const void* vfirst, int ldvf, void* kc, void* vc,
+                  const void* slots, int T_, int H, int G, int D, int DV,
+                  int BS, int dtype, void* stream) {
+  if (T_ <= 0) return;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((attn_prep_kernel<T>), dim3(T_), dim3(256), 0,
+                       (hipStream_t)stream, (T*)q, ldq, (const T*)k, ldk,
+                       (T*)v, ldv, (const float*)qw, (const float*)kw, eps,
+                       (const float*)vmix, (const T*)vfirst, ldvf, (T*)kc,
+                       (T*)vc, (const int64_t*)slots, H, G, D, DV, BS);
+  })
+}
+
+void mx_latent_prep(void* qf, const void* qlat, const void* q, int ldq,
+                    const void* dkv, int lddkv, const void* normw, float eps,
+                    const void* cos_sin, int table_rows, int rot_dims,
+                    const void* positions, void* cache, const void* slots,
+                    int T_, int H, int D, int R, int L, int BS, int dtype,
+                    void* stream) {
+  if (T_ <= 0) return;
+  (void)BS;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((latent_prep_kernel<T>), dim3(T_), dim3(256), 0,
+                       (hipStream_t)stream, (T*)qf, (const T*)qlat,
+                       (const T*)q, ldq, (const T*)dkv, lddkv,
+                       (const float*)normw, eps, (const float*)cos_sin,
+                       table_rows, rot_dims, (const int*)positions,
+                       (T*)cache, (const int64_t*)slots, T_, H, D, R, L, BS);
+  })
+}
+
+#define CONV_CASE(KK)                                                        \
+  case KK:                                                                   \
+    hipLaunchKernelGGL((short_conv_silu_kernel<T, KK>), grid, dim3(256), 0,  \
+                       (hipStream_t)stream, (T*)y, ldy, (const T*)x, ldx,    \
+                       (const float*)w, (T*)state, (const int*)seq_rows, C); \
+    break;
+
+int mx_short_conv_silu(void* y, int ldy, const void* x, int ldx,
+                       const void* w, void* state, const void* seq_rows,
+                       int S_, int C, int K, int T_, int dtype,
+                       void* stream) {
+  if (S_ <= 0 || T_ <= 0) return 0;
+  if (K < 1 || K > 8) return 1;
+  // a segment has at most T_ - (S_ - 1) rows
+  const int longest = T_ - (S_ - 1);
+  dim3 grid((C + 255) / 256, S_, (longest + CONV_CH - 1) / CONV_CH);
+  MX_DISPATCH_DTYPE(dtype, {
+    switch (K) {
+      CONV_CASE(1)
+      CONV_CASE(2)
+      CONV_CASE(3)
+      CONV_CASE(4)
+      CONV_CASE(5)
+      CONV_CASE(6)
+      CONV_CASE(7)
+      CONV_CASE(8)
+    }
+  })
+  return 0;
+}
+
+}  // extern "C"

@@ -1,6 +1,7 @@
 // fp32 residual-stream kernels: scaled embedding gather, fused
-// (residual += deltas) + RMSNorm, gated-MLP inner activations, paged KV
-// append with independent key/value widths.
+// (residual += deltas) + (grouped) RMSNorm, grouped RMSNorm + token shift,
+// depth-weighted sum of residual streams, gated-MLP inner activations, paged
+// KV append with independent key/value widths.
 #include "mix_common.h"
 
 template <typename T>
@@ -13,30 +14,114 @@ __global__ __launch_bounds__(256) void embed_scale_kernel(
     x[(size_t)t * W + c] = MxElem<T>::ld(row + c) * scale;
 }
 
-// x[t] += d0[t] + d1[t] (each optional), h[t] = x[t] / rms(x[t]) * w.
+#define MX_MAX_GROUPS 64
+
+// Per-group 1/rms of one fp32 row into sinv[groups] (LDS); the row is split
+// into `groups` equal consecutive parts. Ends with a barrier.
+PS_DEV void mx_group_inv(const float* __restrict__ xr, int W, int groups,
+                         float eps, float* sinv, float* red) {
+  const int gw = W / groups;
+  for (int g = 0; g < groups; ++g) {
+    float ss = 0.f;
+    for (int c = g * gw + threadIdx.x; c < (g + 1) * gw; c += blockDim.x)
+      ss += xr[c] * xr[c];
+    ss = mx_block_sum(ss, red);
+    if (threadIdx.x == 0) sinv[g] = 1.0f / sqrtf(ss / (float)gw + eps);
+  }
+  __syncthreads();
+}
+
+// xo[t] = xi[t] + d0[t] + d1[t] (each optional; xo may be xi),
+// h[t] = xo[t] / rms(part of xo[t]) * w, one rms per group of W / groups.
 template <typename T>
-__global__ __launch_bounds__(256) void add_rms_norm32_kernel(
-    T* __restrict__ h, float* __restrict__ x, const T* __restrict__ d0,
+__global__ __launch_bounds__(256) void add_group_norm32_kernel(
+    T* __restrict__ h, float* xo, const float* xi, const T* __restrict__ d0,
     int ld0, const T* __restrict__ d1, int ld1, const float* __restrict__ w,
-    float eps, int W) {
+    float eps, int groups, int W) {
   __shared__ float red[17];
+  __shared__ float sinv[MX_MAX_GROUPS];
   const int t = blockIdx.x;
-  float* xr = x + (size_t)t * W;
-  float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float v = xr[c];
-    if (d0 != nullptr) {
-      float d = MxElem<T>::ld(d0 + (size_t)t * ld0 + c);
-      if (d1 != nullptr) d += MxElem<T>::ld(d1 + (size_t)t * ld1 + c);
-      v += d;
+  float* xr = xo + (size_t)t * W;
+  const float* xs = xi + (size_t)t * W;
+  if (d0 != nullptr || xo != xi) {
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      float v = xs[c];
+      if (d0 != nullptr) {
+        float d = MxElem<T>::ld(d0 + (size_t)t * ld0 + c);
+        if (d1 != nullptr) d += MxElem<T>::ld(d1 + (size_t)t * ld1 + c);
+        v += d;
+      }
       xr[c] = v;
     }
-    ss += v * v;
+    __syncthreads();  // the sums below read other threads' entries
   }
-  ss = mx_block_sum(ss, red);
-  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  mx_group_inv(xr, W, groups, eps, sinv, red);
+  const int gw = W / groups;
   for (int c = threadIdx.x; c < W; c += blockDim.x)
-    MxElem<T>::st(h + (size_t)t * W + c, xr[c] * inv * w[c]);
+    MxElem<T>::st(h + (size_t)t * W + c, xr[c] * sinv[c / gw] * w[c]);
+}
+
+// Grouped RMSNorm + token shift. With hn(r) = x[r] / rms * w, row t gets
+//   h[t] = hn(t) + (prev - hn(t)) * shift,
+// prev = hn(t - 1) inside a segment, state[slot] for its first row (zeros at
+// position 0). The workgroup of a segment's first row is the only one that
+// reads state[slot], and it writes the segment's last hn there afterwards
+// (same thread per channel), so no other workgroup races with it.
+template <typename T>
+__global__ __launch_bounds__(256) void group_norm_shift_kernel(
+    T* __restrict__ h, const float* __restrict__ x,
+    const float* __restrict__ w, float eps, int groups,
+    const float* __restrict__ shift, float* __restrict__ state,
+    const int* __restrict__ token_seq, const int* __restrict__ seq_rows,
+    int W) {
+  __shared__ float red[17];
+  __shared__ float sinv[3][MX_MAX_GROUPS];
+  const int t = blockIdx.x;
+  const int* sr = seq_rows + 4 * token_seq[t];
+  const int t0 = sr[0], n = sr[1], p0 = sr[2], slot = sr[3];
+  const bool first = t == t0;
+  const int last = t0 + n - 1;
+  const float* xr = x + (size_t)t * W;
+  const float* xp = x + (size_t)(first ? t : t - 1) * W;
+  const float* xl = x + (size_t)last * W;
+  mx_group_inv(xr, W, groups, eps, sinv[0], red);
+  if (!first) mx_group_inv(xp, W, groups, eps, sinv[1], red);
+  if (first && n > 1) mx_group_inv(xl, W, groups, eps, sinv[2], red);
+  const int gw = W / groups;
+  float* st = state + (size_t)slot * W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const int g = c / gw;
+    const float hn = xr[c] * sinv[0][g] * w[c];
+    float prev;
+    if (!first) {
+      prev = xp[c] * sinv[1][g] * w[c];
+    } else {
+      prev = p0 > 0 ? st[c] : 0.f;
+      st[c] = n > 1 ? xl[c] * sinv[2][g] * w[c] : hn;
+    }
+    MxElem<T>::st(h + (size_t)t * W + c, hn + (prev - hn) * shift[c]);
+  }
+}
+
+// Newest stream = base + delta, stored at hist[n-1]; out = sum_j wts[j] *
+// hist[j] over the n streams (fp32, ascending j).
+template <typename T>
+__global__ __launch_bounds__(256) void depth_mix_kernel(
+    float* __restrict__ out, float* hist, int n,
+    const float* __restrict__ wts, const float* base,
+    const T* __restrict__ delta, int ldd, int T_, int W) {
+  const size_t TS = (size_t)T_ * W;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < TS;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / W;
+    const int c = (int)(idx - t * W);
+    const float nw = base[idx] + MxElem<T>::ld(delta + t * ldd + c);
+    float acc = 0.f;
+    for (int j = 0; j < n - 1; ++j) acc += wts[j] * hist[j * TS + idx];
+    acc += wts[n - 1] * nw;
+    hist[(size_t)(n - 1) * TS + idx] = nw;
+    out[idx] = acc;
+  }
 }
 
 #define MX_ACT_SILU 0
@@ -99,14 +184,54 @@ void mx_embed_scale(void* x, const void* tokens, const void* embed,
   })
 }
 
+void mx_add_group_norm32(void* h, void* xo, const void* xi, const void* d0,
+                         int ld0, const void* d1, int ld1, const void* w,
+                         float eps, int groups, int T_, int W, int dtype,
+                         void* stream) {
+  if (T_ <= 0) return;
+  if (groups < 1 || groups > MX_MAX_GROUPS || W % groups) return;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((add_group_norm32_kernel<T>), dim3(T_), dim3(256), 0,
+                       (hipStream_t)stream, (T*)h, (float*)xo,
+                       (const float*)xi, (const T*)d0, ld0, (const T*)d1,
+                       ld1, (const float*)w, eps, groups, W);
+  })
+}
+
 void mx_add_rms_norm32(void* h, void* x, const void* d0, int ld0,
                        const void* d1, int ld1, const void* w, float eps,
                        int T_, int W, int dtype, void* stream) {
+  mx_add_group_norm32(h, x, x, d0, ld0, d1, ld1, w, eps, 1, T_, W, dtype,
+                      stream);
+}
+
+void mx_group_norm_shift(void* h, const void* x, const void* w, float eps,
+                         int groups, const void* shift, void* state,
+                         const void* token_seq, const void* seq_rows, int T_,
+                         int W, int dtype, void* stream) {
   if (T_ <= 0) return;
+  if (groups < 1 || groups > MX_MAX_GROUPS || W % groups) return;
   MX_DISPATCH_DTYPE(dtype, {
-    hipLaunchKernelGGL((add_rms_norm32_kernel<T>), dim3(T_), dim3(256), 0,
-                       (hipStream_t)stream, (T*)h, (float*)x, (const T*)d0,
-                       ld0, (const T*)d1, ld1, (const float*)w, eps, W);
+    hipLaunchKernelGGL((group_norm_shift_kernel<T>), dim3(T_), dim3(256), 0,
+                       (hipStream_t)stream, (T*)h, (const float*)x,
+                       (const float*)w, eps, groups, (const float*)shift,
+                       (float*)state, (const int*)token_seq,
+                       (const int*)seq_rows, W);
+  })
+}
+
+void mx_depth_mix(void* out, void* hist, int n, const void* wts,
+                  const void* base, const void* delta, int ldd, int T_, int W,
+                  int dtype, void* stream) {
+  if (T_ <= 0 || n < 1) return;
+  const size_t total = (size_t)T_ * W;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((depth_mix_kernel<T>), dim3((unsigned)blocks),
+                       dim3(256), 0, (hipStream_t)stream, (float*)out,
+                       (float*)hist, n, (const float*)wts,
+                       (const float*)base, (const T*)delta, ldd, T_, W);
   })
 }
 

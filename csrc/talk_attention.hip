@@ -1,5 +1,9 @@
 // Paged attention with head-mixed ("talking") scores, aligned-chunk and
-// trailing-window visibility, and an optional denominator sink.
+// trailing-window visibility (optionally keeping a sequence's first keys
+// visible behind the window), capped scores and an optional denominator
+// sink (score 0 or a learned per-head score). The values may be the leading
+// entries of wider cache rows, so keys that carry their values (latent
+// attention) need one cache.
 //
 // One launch covers a ragged batch: every token carries (its sequence's
 // block-table row, its position); keys and values come from the paged
@@ -14,6 +18,21 @@
 #include "mix_common.h"
 
 #define TA_KT 32
+
+// Options beyond the basic shape. keep_first: keys [0, keep_first) stay
+// visible to every later query; softcap > 0: score <- cap * tanh(score /
+// cap), after the head mix; sink_vals: per-head sink scores (nullptr: 0);
+// vr: elements per row of the value cache (>= DV).
+struct TaOpt {
+  int keep_first;
+  float softcap;
+  const float* sink_vals;
+  int vr;
+};
+
+PS_DEV float ta_cap(float sc, float cap) {
+  return cap > 0.f ? cap * tanhf(sc / cap) : sc;
+}
 
 // Dynamic LDS a kernel may ask for: gfx950 has 160 KB per CU, but a launch
 // above 64 KB needs the limit raised per kernel first. Falls back to 64 KB
@@ -34,7 +53,7 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
     const float* __restrict__ talk, int H, int G, int D, int DV, int BS,
-    float scale, int chunk, int window, int sink) {
+    float scale, int chunk, int window, int sink, TaOpt opt) {
   extern __shared__ float lds[];
   float* sq = lds;                 // [H*D]
   float* ss = sq + H * D;          // [H][KT] raw scores
@@ -59,13 +78,17 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
   if (talk != nullptr)
     for (int c = threadIdx.x; c < H * H; c += blockDim.x) stk[c] = talk[c];
   for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    sm[h] = sink ? 0.f : PS_NEG_INF;
+    sm[h] = sink ? (opt.sink_vals ? opt.sink_vals[h] : 0.f) : PS_NEG_INF;
     sl[h] = sink ? 1.f : 0.f;
   }
   __syncthreads();
 
-  for (int j0 = lo; j0 <= pos; j0 += TA_KT) {
-    const int nk = min(TA_KT, pos + 1 - j0);
+  // two key ranges: the kept first keys behind the window, then the window
+  for (int rg = 0; rg < 2; ++rg) {
+  const int ra = rg == 0 ? 0 : lo;
+  const int rb = rg == 0 ? min(opt.keep_first, lo) - 1 : pos;
+  for (int j0 = ra; j0 <= rb; j0 += TA_KT) {
+    const int nk = min(TA_KT, rb + 1 - j0);
     // raw scores of every (head, key) pair of the tile
     for (int it = threadIdx.x; it < H * nk; it += blockDim.x) {
       const int jj = it / H, h = it % H;
@@ -89,7 +112,7 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
       } else {
         m = ss[h * TA_KT + jj];
       }
-      sp[h * TA_KT + jj] = m;
+      sp[h * TA_KT + jj] = ta_cap(m, opt.softcap);
     }
     __syncthreads();
     // online softmax bookkeeping: one thread per head
@@ -118,11 +141,12 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
         const int64_t blk = table[j / BS];
         acc += sp[h * TA_KT + jj] *
                MxElem<T>::ld(vc + ((blk * G + gk) * BS + (j % BS)) *
-                                      (int64_t)DV + d);
+                                      (int64_t)opt.vr + d);
       }
       sacc[it] = acc;
     }
     __syncthreads();
+  }
   }
   for (int it = threadIdx.x; it < H * DV; it += blockDim.x)
     MxElem<T>::st(out + (size_t)t * ldout + it, sacc[it] / sl[it / DV]);
@@ -163,11 +187,12 @@ struct TaVec<mx_bf16> {
 template <typename T, int DP, int PITCH>
 PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
                      const int* __restrict__ table, int j0, int nk, int G,
-                     int Dw, int BS) {
+                     int Dw, int BS, int RW) {
+  // Dw elements of every cache row of RW elements are staged
   constexpr int VEC = TaVec<T>::N;
   constexpr int U = 8;
   const int tid = threadIdx.x, nt = blockDim.x;
-  if (Dw % VEC == 0) {
+  if (Dw % VEC == 0 && RW % VEC == 0) {
     const int vpr = Dw / VEC;
     const int total = nk * G * vpr;
     for (int base = 0; base < total; base += nt * U) {
@@ -182,7 +207,7 @@ PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
           const int jj = row / G, g = row - jj * G;
           const int j = j0 + jj;
           const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-          buf[u] = *(const float4*)(cache + gb * Dw + c * VEC);
+          buf[u] = *(const float4*)(cache + gb * RW + c * VEC);
           off[u] = row * PITCH + c * VEC;
         }
       }
@@ -203,7 +228,7 @@ PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
       const int jj = row / G, g = row - jj * G;
       const int j = j0 + jj;
       const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-      sdst[row * PITCH + d] = d < Dw ? MxElem<T>::ld(cache + gb * Dw + d) : 0.f;
+      sdst[row * PITCH + d] = d < Dw ? MxElem<T>::ld(cache + gb * RW + d) : 0.f;
     }
   }
 }
@@ -227,7 +252,8 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
     const float* __restrict__ talk, int T_total, int H, int G, int D, int DV,
-    int BS, float scale, int chunk, int window, int sink, int QT, int KT) {
+    int BS, float scale, int chunk, int window, int sink, int QT, int KT,
+    TaOpt opt) {
   extern __shared__ float lds[];
   const int NP = H * QT;
   float* sK = lds;                   // [KT][G][DP]
@@ -261,7 +287,8 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
                 : 0.f;
     acc[d] = 0.f;
   }
-  float m = sink ? 0.f : PS_NEG_INF;
+  float m = sink ? ((opt.sink_vals && valid) ? opt.sink_vals[h] : 0.f)
+                 : PS_NEG_INF;
   float l = sink ? 1.f : 0.f;
   __syncthreads();
   const int my_pos = valid ? s_pos[i] : 0;
@@ -282,11 +309,15 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
     if (window > 0) kmin = max(kmin, s_pos[rs] - window + 1);
     const int kmax = s_pos[re - 1];
 
-    for (int j0 = kmin; j0 <= kmax; j0 += KT) {
-      const int nk = min(KT, kmax + 1 - j0);
+    // kept first keys behind the run's earliest window, then the windows
+    for (int rg = 0; rg < 2; ++rg) {
+    const int ra = rg == 0 ? 0 : kmin;
+    const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1 : kmax;
+    for (int j0 = ra; j0 <= rb; j0 += KT) {
+      const int nk = min(KT, rb + 1 - j0);
       __syncthreads();  // the previous tile is fully consumed
-      ta_stage<T, DP, DP>(sK, kc, table, j0, nk, G, D, BS);
-      ta_stage<T, DP, DP>(sV, vc, table, j0, nk, G, DV, BS);
+      ta_stage<T, DP, DP>(sK, kc, table, j0, nk, G, D, BS, D);
+      ta_stage<T, DP, DP>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
       __syncthreads();
       if (mine) {
         for (int jj = 0; jj < nk; ++jj) {
@@ -316,8 +347,10 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
           } else {
             sc = sS[jj * NP + tid];
           }
+          sc = ta_cap(sc, opt.softcap);
           const int j = j0 + jj;
-          if (j > my_pos || j < my_lo) sc = PS_NEG_INF;
+          if (j > my_pos || (j < my_lo && j >= opt.keep_first))
+            sc = PS_NEG_INF;
           sM[jj * NP + tid] = sc;
           mx = fmaxf(mx, sc);
         }
@@ -348,6 +381,7 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
         }
       }
     }
+    }
     rs = re;
   }
   if (valid) {
@@ -366,7 +400,7 @@ static int launch_tiled(void* out, int ldout, const void* q, int ldq,
                         const void* token_seq, const void* token_pos,
                         const void* talk, int T_, int H, int G, int D, int DV,
                         int BS, float scale, int chunk, int window, int sink,
-                        hipStream_t stream) {
+                        TaOpt opt, hipStream_t stream) {
   static const size_t budget =
       ta_lds_budget((const void*)talk_attn_tiled_kernel<T, DP>);
   const int QT = 256 / H, NP = H * QT;
@@ -384,7 +418,7 @@ static int launch_tiled(void* out, int ldout, const void* q, int ldq,
                      (const T*)vc, (const int*)block_tables, max_blocks,
                      (const int*)token_seq, (const int*)token_pos,
                      (const float*)talk, T_, H, G, D, DV, BS, scale, chunk,
-                     window, sink, QT, KT);
+                     window, sink, QT, KT, opt);
   return 0;
 }
 
@@ -405,7 +439,7 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
     const float* __restrict__ talk, int H, int G, int D, int DV, int BS,
     float scale, int chunk, int window, int sink, int NS, int KPT, int KS,
-    float* __restrict__ part) {
+    float* __restrict__ part, TaOpt opt) {
   extern __shared__ float lds[];
   constexpr int PITCH = DP + 4;
   const int TK = NS * KPT;           // keys per tile
@@ -427,6 +461,8 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   int lo = 0, pos = token_pos[t];
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
+  // the kept first keys behind the window go to share 0
+  const int kept = ks == 0 ? min(opt.keep_first, lo) : 0;
   if (KS > 1) {
     // this workgroup's share of the visible keys, in whole tiles
     const int tiles = (pos + 1 - lo + TK - 1) / TK;
@@ -449,14 +485,18 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
 #pragma unroll
   for (int d = 0; d < DP; ++d) acc[d] = 0.f;
   const bool own_sink = sink && i == 0 && ks == 0;
-  float m = own_sink ? 0.f : PS_NEG_INF;
+  float m = own_sink ? ((opt.sink_vals && valid) ? opt.sink_vals[h] : 0.f)
+                     : PS_NEG_INF;
   float l = own_sink ? 1.f : 0.f;
 
-  for (int j0 = lo; j0 <= pos; j0 += TK) {
-    const int nk = min(TK, pos + 1 - j0);
+  for (int rg = 0; rg < 2; ++rg) {
+  const int ra = rg == 0 ? 0 : lo;
+  const int rb = rg == 0 ? kept - 1 : pos;
+  for (int j0 = ra; j0 <= rb; j0 += TK) {
+    const int nk = min(TK, rb + 1 - j0);
     __syncthreads();
-    ta_stage<T, DP, PITCH>(sK, kc, table, j0, nk, G, D, BS);
-    ta_stage<T, DP, PITCH>(sV, vc, table, j0, nk, G, DV, BS);
+    ta_stage<T, DP, PITCH>(sK, kc, table, j0, nk, G, D, BS, D);
+    ta_stage<T, DP, PITCH>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
     __syncthreads();
     if (valid) {
       for (int c = 0; c < KPT; ++c) {
@@ -491,6 +531,7 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
           } else {
             sc = sS[jj * H + h];
           }
+          sc = ta_cap(sc, opt.softcap);
           const float mx = fmaxf(m, sc);
           const float alpha = expf(m - mx);  // m = -inf gives 0
           const float p = expf(sc - mx);
@@ -508,6 +549,7 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
         }
       }
     }
+  }
   }
   // merge the NS slices of each head
   __syncthreads();
@@ -588,7 +630,7 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
                         const void* token_seq, const void* token_pos,
                         const void* talk, int T_, int H, int G, int D, int DV,
                         int BS, float scale, int chunk, int window, int sink,
-                        hipStream_t stream, int KS, float* part) {
+                        TaOpt opt, hipStream_t stream, int KS, float* part) {
   static const size_t budget =
       ta_lds_budget((const void*)talk_attn_split_kernel<T, DP>);
   if (KS < 1 || part == nullptr) KS = 1;
@@ -616,7 +658,7 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
                      (const T*)kc, (const T*)vc, (const int*)block_tables,
                      max_blocks, (const int*)token_seq,
                      (const int*)token_pos, (const float*)talk, H, G, D, DV,
-                     BS, scale, chunk, window, sink, NS, KPT, KS, part);
+                     BS, scale, chunk, window, sink, NS, KPT, KS, part, opt);
   if (KS > 1)
     hipLaunchKernelGGL((talk_attn_combine_kernel<T>), dim3(T_), dim3(256), 0,
                        stream, (T*)out, ldout, (const float*)part, H, DV, KS);
@@ -628,17 +670,17 @@ static int launch_split(void* out, int ldout, const void* q, int ldq,
     if (dmax <= 32)                                                          \
       rc = FN<T, 32>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
                      token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
-                     chunk, window, sink, (hipStream_t)stream,               \
+                     chunk, window, sink, opt, (hipStream_t)stream,               \
                      ##__VA_ARGS__);                                         \
     else if (dmax <= 64)                                                     \
       rc = FN<T, 64>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,   \
                      token_seq, token_pos, talk, T_, H, G, D, DV, BS, scale, \
-                     chunk, window, sink, (hipStream_t)stream,               \
+                     chunk, window, sink, opt, (hipStream_t)stream,               \
                      ##__VA_ARGS__);                                         \
     else                                                                     \
       rc = FN<T, 128>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,  \
                       token_seq, token_pos, talk, T_, H, G, D, DV, BS,       \
-                      scale, chunk, window, sink, (hipStream_t)stream,       \
+                      scale, chunk, window, sink, opt, (hipStream_t)stream,       \
                       ##__VA_ARGS__);                                        \
   })
 
@@ -653,8 +695,13 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                                  int T_, int H, int G, int D, int DV, int BS,
                                  float scale, int chunk, int window,
                                  int sink, int dtype, int variant,
-                                 int splits, void* scratch, void* stream) {
+                                 int splits, void* scratch, int keep_first,
+                                 float softcap, const void* sink_vals,
+                                 int vrow, void* stream) {
   if (T_ <= 0) return 0;
+  if (vrow < DV) return 3;
+  const TaOpt opt = {keep_first > 0 ? keep_first : 0, softcap,
+                     (const float*)sink_vals, vrow};
   const int dmax = D > DV ? D : DV;
   if ((variant == 0 || variant == 2) && H <= 256 && dmax <= 128) {
     int rc = 1;
@@ -677,7 +724,7 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                        (const T*)kc, (const T*)vc, (const int*)block_tables,
                        max_blocks, (const int*)token_seq,
                        (const int*)token_pos, (const float*)talk, H, G, D, DV,
-                       BS, scale, chunk, window, sink);
+                       BS, scale, chunk, window, sink, opt);
   })
   return 0;
 }

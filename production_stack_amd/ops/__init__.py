@@ -485,7 +485,7 @@ def add_rms_norm32(x32: torch.Tensor, deltas, w32: torch.Tensor, eps: float,
     T, W = x32.shape
     assert x32.dtype == torch.float32 and x32.is_contiguous()
     assert w32.dtype == torch.float32 and w32.numel() == W
-    assert groups >= 1 and W % groups == 0
+    assert 1 <= groups <= 64 and W % groups == 0
     if out32 is None:
         out32 = x32
     assert out32.dtype == torch.float32 and out32.is_contiguous()
@@ -528,7 +528,8 @@ def group_norm_shift(x32: torch.Tensor, w32: torch.Tensor, eps: float,
     assert w32.dtype == torch.float32 and w32.numel() == W
     assert shift.dtype == torch.float32 and shift.numel() == W
     assert state.dtype == torch.float32 and state.shape[1:] == (W,)
-    assert state.is_contiguous() and W % groups == 0
+    assert state.is_contiguous() and 1 <= groups <= 64
+    assert W % groups == 0
     assert token_seq.dtype == torch.int32 and token_seq.shape == (T,)
     _check_seq_rows(seq_rows)
     h = torch.empty((T, W), dtype=out_dtype, device=x32.device)

@@ -1,7 +1,8 @@
 """Builder and loader of the mixer-kernel library (`_mixops.so`).
 
-The fp32-residual / delta-rule / talking-attention kernels (csrc/resid32.hip,
-csrc/delta_rule.hip, csrc/talk_attention.hip) expose a plain C ABI, so the
+The fp32-residual / delta-rule / attention kernels (csrc/resid32.hip,
+csrc/delta_rule.hip, csrc/gated_delta.hip, csrc/talk_attention.hip,
+csrc/mixer_prep.hip) expose a plain C ABI, so the
 library needs hipcc only: no torch headers, seconds-to-minutes to build, and
 a fresh checkout can compile just these files on first use without building
 the large `_C` extension. Launchers receive raw device pointers and the
@@ -35,6 +36,9 @@ UNITS = [
     ("talk_attention.hip", []),
     ("delta_rule.hip", ["-DMX_ONLY_DTYPE=0"]),
     ("delta_rule.hip", ["-DMX_ONLY_DTYPE=1"]),
+    ("mixer_prep.hip", []),
+    ("gated_delta.hip", ["-DMX_ONLY_DTYPE=0"]),
+    ("gated_delta.hip", ["-DMX_ONLY_DTYPE=1"]),
 ]
 
 _lib = None
@@ -89,10 +93,13 @@ def load():
         if not os.path.exists(LIB_PATH):
             build()
         lib = ctypes.CDLL(LIB_PATH)
-        for name in ("mx_delta_rule", "mx_talk_attention"):
+        for name in ("mx_delta_rule", "mx_talk_attention",
+                     "mx_gated_delta", "mx_short_conv_silu"):
             getattr(lib, name).restype = ctypes.c_int
-        for name in ("mx_embed_scale", "mx_add_rms_norm32", "mx_gated_act",
-                     "mx_kv_append"):
+        for name in ("mx_embed_scale", "mx_add_rms_norm32",
+                     "mx_add_group_norm32", "mx_group_norm_shift",
+                     "mx_depth_mix", "mx_gated_act", "mx_kv_append",
+                     "mx_attn_prep", "mx_latent_prep"):
             getattr(lib, name).restype = None
         _lib = lib
     return _lib
