@@ -474,6 +474,78 @@ ARCHITECTURES.update({
 })
 
 
+def _derusun_stack(
+    name: str, width: int, vocab: int, n_layers: int, *, delta_heads: int,
+    delta_kv: int, delta_dim: int, delta_vdim: int, conv: int, rank: int,
+    attn_heads: int, attn_kv: int, attn_dim: int, window: int,
+    keep_first: int, softcap: float, lat_heads: int, lat_dim: int,
+    lat_rot: int, lat_vdim: int, kv_rank: int, ff: int, limit: float = 7.0,
+    groups: int = 4,
+) -> ModelConfig:
+    """A Derusun stack in the repeating order channel-delta, windowed
+    attention, channel-delta, latent attention; sequential sublayers, every
+    layer with a dense clamped-swish feed-forward, token shift and
+    depth-weighted streams; all windowed layers mix values."""
+    specs = []
+    for i in range(n_layers):
+        k = i % 4
+        if k in (0, 2):
+            mixer = MixerSpec(
+                kind="channel_delta", heads=delta_heads, kv_heads=delta_kv,
+                dim=delta_dim, vdim=delta_vdim, conv=conv, decay_rank=rank,
+                gate_rank=rank, rope=False)
+        elif k == 1:
+            mixer = MixerSpec(
+                kind="attention", heads=attn_heads, kv_heads=attn_kv,
+                dim=attn_dim, vdim=attn_dim, scale=attn_dim ** -0.5,
+                window=window, keep_first=keep_first, softcap=softcap,
+                sink=True, learned_sink=True, bias=True, qk_norm=True,
+                v_mix=True, rope=False)
+        else:
+            mixer = MixerSpec(
+                kind="latent_attention", heads=lat_heads, kv_heads=1,
+                dim=lat_dim, vdim=lat_vdim, kv_rank=kv_rank,
+                rot_dim=lat_rot, rot_dims=lat_rot, rot_base=1e6,
+                scale=(lat_dim + lat_rot) ** -0.5, sink=True,
+                learned_sink=True, rope=True)
+        specs.append(LayerSpec(
+            mixer=mixer,
+            mlp=MlpSpec(kind="dense", ff=ff, act="clamped_swish",
+                        limit=limit),
+            parallel=False, token_shift=True, depth_average=True))
+    return ModelConfig(
+        name=name, family="derusun", hidden_size=width,
+        num_layers=n_layers, num_q_heads=attn_heads, num_kv_heads=attn_kv,
+        head_dim=attn_dim, intermediate_size=ff, vocab_size=vocab,
+        max_position=8192, layer_specs=specs, norm_groups=groups,
+        bos_token_id=0, eos_token_id=-1)
+
+
+ARCHITECTURES.update({
+    # CPU-runnable test config
+    "tiny-derusun": _derusun_stack(
+        "tiny-derusun", 96, 384, 4, delta_heads=4, delta_kv=2,
+        delta_dim=16, delta_vdim=24, conv=3, rank=8, attn_heads=6,
+        attn_kv=3, attn_dim=16, window=40, keep_first=2, softcap=10.0,
+        lat_heads=4, lat_dim=16, lat_rot=8, lat_vdim=12, kv_rank=24,
+        ff=160, limit=2.0, groups=3),
+    # llama-3.2-1b-sized stack (same width, depth, ff and vocab)
+    "derusun-1b": _derusun_stack(
+        "derusun-1b", 2048, 128256, 16, delta_heads=32, delta_kv=16,
+        delta_dim=64, delta_vdim=64, conv=4, rank=64, attn_heads=32,
+        attn_kv=8, attn_dim=64, window=1024, keep_first=4, softcap=30.0,
+        lat_heads=32, lat_dim=64, lat_rot=32, lat_vdim=64, kv_rank=256,
+        ff=8192),
+    # llama-3-8b-sized layers (width 4096, head dim 128, ff 14336)
+    "derusun-8b": _derusun_stack(
+        "derusun-8b", 4096, 128256, 32, delta_heads=32, delta_kv=16,
+        delta_dim=128, delta_vdim=128, conv=4, rank=128, attn_heads=32,
+        attn_kv=8, attn_dim=128, window=2048, keep_first=4, softcap=30.0,
+        lat_heads=32, lat_dim=128, lat_rot=64, lat_vdim=128, kv_rank=512,
+        ff=14336),
+})
+
+
 @dataclass
 class CacheConfig:
     block_size: int = 16

@@ -139,7 +139,7 @@ def attention(h, W, pre, m, eps, v_first=None):
     k = group_rms_norm(k, W[pre + "k.norm"], eps)
     if m.get("v_mix") and v_first is not None:
         lam = W[pre + "vmix"].to(F64)
-        v = (1.0 - lam) * v + lam * v_first
+        v = (1.0 - lam) * v + lam * v_first.to(F64)
     kk = k.repeat_interleave(rep, dim=1)
     vv = v.repeat_interleave(rep, dim=1)
     s = torch.einsum("ihd,jhd->hij", q, kk) * m["scale"]
