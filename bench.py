@@ -114,6 +114,7 @@ class User:
 # closest Llama config at equal width, depth, dense-ff width and vocabulary
 COMPARE_PAIRS = {
     "nanurax": [("nanurax-1b", "llama-3.2-1b"), ("nanurax-8b", "llama-3-8b")],
+    "derusun": [("derusun-1b", "llama-3.2-1b"), ("derusun-8b", "llama-3-8b")],
 }
 
 

@@ -52,9 +52,18 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
     const T* __restrict__ kc, const T* __restrict__ vc,
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
-    const float* __restrict__ talk, int H, int G, int D, int DV, int BS,
-    float scale, int chunk, int window, int sink, TaOpt opt) {
+    const float* __restrict__ talk, int HT, int G, int D, int DV, int BS,
+    float scale, int chunk, int window, int sink, TaOpt opt, int HB) {
+  // Without a head mix the heads are independent: a workgroup then takes
+  // the HB heads from blockIdx.y * HB on (HT heads in all), which bounds
+  // the LDS need for wide heads. With a mix HB == HT.
   extern __shared__ float lds[];
+  const int h0 = blockIdx.y * HB;
+  const int H = min(HB, HT - h0);
+  const int rep = HT / G;
+  q += h0 * D;
+  out += h0 * DV;
+  if (opt.sink_vals) opt.sink_vals += h0;
   float* sq = lds;                 // [H*D]
   float* ss = sq + H * D;          // [H][KT] raw scores
   float* sp = ss + H * TA_KT;      // [H][KT] mixed scores -> weights
@@ -70,7 +79,6 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
-  const int rep = H / G;
 
   for (int c = threadIdx.x; c < H * D; c += blockDim.x)
     sq[c] = MxElem<T>::ld(q + (size_t)t * ldq + c);
@@ -94,7 +102,8 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
       const int jj = it / H, h = it % H;
       const int j = j0 + jj;
       const int64_t blk = table[j / BS];
-      const T* kr = kc + ((blk * G + h / rep) * BS + (j % BS)) * (int64_t)D;
+      const T* kr =
+          kc + ((blk * G + (h0 + h) / rep) * BS + (j % BS)) * (int64_t)D;
       const float* qh = sq + h * D;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc += qh[d] * MxElem<T>::ld(kr + d);
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
     // P.V
     for (int it = threadIdx.x; it < H * DV; it += blockDim.x) {
       const int h = it / DV, d = it % DV;
-      const int gk = h / rep;
+      const int gk = (h0 + h) / rep;
       float acc = sacc[it] * sal[h];
       for (int jj = 0; jj < nk; ++jj) {
         const int j = j0 + jj;
@@ -714,17 +723,25 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
     if (rc == 0) return 0;
   }
   if (variant == 2 || variant == 4) return 2;
-  const size_t lds =
-      (size_t)(H * D + 2 * H * TA_KT + H * DV + 3 * H + H * H) *
-      sizeof(float);
+  // heads per workgroup: all of them with a head mix, otherwise as many as
+  // fit 64 KB of LDS
+  int HB = H;
+  auto need = [&](int hb) {
+    return (size_t)(hb * D + 2 * hb * TA_KT + hb * DV + 3 * hb +
+                    (talk != nullptr ? H * H : 0)) * sizeof(float);
+  };
+  if (talk == nullptr)
+    while (HB > 1 && need(HB) > 64 * 1024) HB = (HB + 1) / 2;
+  const size_t lds = need(HB);
   if (lds > 64 * 1024) return 1;
   MX_DISPATCH_DTYPE(dtype, {
-    hipLaunchKernelGGL((talk_attn_kernel<T>), dim3(T_), dim3(256), lds,
-                       (hipStream_t)stream, (T*)out, ldout, (const T*)q, ldq,
-                       (const T*)kc, (const T*)vc, (const int*)block_tables,
-                       max_blocks, (const int*)token_seq,
-                       (const int*)token_pos, (const float*)talk, H, G, D, DV,
-                       BS, scale, chunk, window, sink, opt);
+    hipLaunchKernelGGL((talk_attn_kernel<T>), dim3(T_, (H + HB - 1) / HB),
+                       dim3(256), lds, (hipStream_t)stream, (T*)out, ldout,
+                       (const T*)q, ldq, (const T*)kc, (const T*)vc,
+                       (const int*)block_tables, max_blocks,
+                       (const int*)token_seq, (const int*)token_pos,
+                       (const float*)talk, H, G, D, DV, BS, scale, chunk,
+                       window, sink, opt, HB);
   })
   return 0;
 }

@@ -622,7 +622,9 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     variant 0 picks the kernel for prompt portions (tiled thread-per-
     (head, query) where the shape fits), 3 for single tokens (split-key),
     both falling back to the plain one-workgroup-per-token kernel; 1 / 2 /
-    4 force plain / tiled / split-key.
+    4 force plain / tiled / split-key. bfloat16 batches without head mix
+    and aligned chunks take the matrix-core kernel instead when the shape
+    fits it (variants 0 and 3; 5 insists on it).
     Returns [T, H*DV]."""
     NB, G, BS, D = k_cache.shape
     VR = v_cache.shape[3]
@@ -658,13 +660,31 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     # workgroup per token, each token's keys are shared out over several
     # workgroups whose partial softmax records are merged afterwards
     scratch = None
-    if variant not in (3, 4):
+    if variant not in (3, 4, 5):
         splits = 1
     elif splits <= 0:
-        splits = max(1, min(8, 512 // T)) if T < 256 else 1
+        splits = (max(1, min(8, 512 // T))
+                  if T < 256 and variant != 5 else 1)
     if splits > 1:
         scratch = torch.empty((T, splits, H, DV + 2),
                               dtype=torch.float32, device=q.device)
+    # bf16 without head mix / aligned chunks: the matrix-core kernel, where
+    # the shape fits it (variant 5 insists on it)
+    if (variant in (0, 3, 5) and q.dtype == torch.bfloat16 and talk is None
+            and chunk == 0):
+        rc = _mx().mx_mfma_attention(
+            _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
+            _p(v_cache), _p(block_tables), block_tables.shape[1],
+            _p(token_seq), _p(token_pos), T, H, G, D, DV, BS, _f(scale),
+            int(window), int(bool(sink)), int(keep_first), _f(softcap),
+            _p(sink_vals), int(VR),
+            int(v_cache.data_ptr() == k_cache.data_ptr()), int(splits),
+            _p(scratch), _stream())
+        if rc == 0:
+            return out
+    if variant == 5:
+        raise RuntimeError(
+            "talk_attention: shape or dtype outside the matrix-core kernel")
     rc = _mx().mx_talk_attention(
         _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
         _p(v_cache), _p(block_tables), block_tables.shape[1],

@@ -459,7 +459,8 @@ def oracle_attend(q, k, v, scale, size, keep, cap, sink):
                         v.double().repeat_interleave(rep, 1)), p
 
 
-def paged(q, k, v, device, bs=16, sizes=(None,), variant_last=None, **kw):
+def paged(q, k, v, device, bs=16, sizes=(None,), variant_last=None,
+          dtype=torch.float32, **kw):
     """Run ops.talk_attention over a scattered paged cache, in portions;
     the last portion may force a kernel variant."""
     T, H, D = q.shape
@@ -467,8 +468,9 @@ def paged(q, k, v, device, bs=16, sizes=(None,), variant_last=None, **kw):
     per = (T + bs - 1) // bs
     g = torch.Generator().manual_seed(7)
     table = torch.randperm(per + 3, generator=g)[:per].to(torch.int32)
-    kc = torch.randn(per + 3, G, bs, D, generator=g).to(device)
-    vc = torch.randn(per + 3, G, bs, DV, generator=g).to(device)
+    kc = torch.randn(per + 3, G, bs, D, generator=g).to(dtype).to(device)
+    vc = torch.randn(per + 3, G, bs, DV, generator=g).to(dtype).to(device)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
     outs = []
     cc = cuts(T, sizes)
     for n, (a, b) in enumerate(cc):
@@ -485,7 +487,7 @@ def paged(q, k, v, device, bs=16, sizes=(None,), variant_last=None, **kw):
             table[None].to(device),
             torch.zeros(b - a, dtype=torch.int32, device=device),
             pos.to(device), heads=H, variant=variant, **kw))
-    return torch.cat(outs).view(T, H, DV)
+    return torch.cat(outs).view(T, H, DV).float()
 
 
 NEEDLE_MODES = [((None,), None), ((None,), 1), ((0, 1), None), ((0, 1), 4),
@@ -574,3 +576,75 @@ def test_values_read_from_key_rows(device):
         assert got.shape == (T, H * DV)
         assert rel_err(got, want.reshape(T, -1)) < 1e-4, variant
     assert per * bs >= T and not math.isnan(float(got.sum()))
+
+
+# ---------------------------------------------------------------------------
+# the matrix-core kernel (bfloat16 on the GPU only)
+# ---------------------------------------------------------------------------
+def bf(x):
+    return x.to(torch.bfloat16).float()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode,splits", [((None,), 0), ((0, 1), 0),
+                                         ((0, 1), 3), ((0, 2), 0),
+                                         ((0, 7), 0)])
+@pytest.mark.parametrize("T,size,keep,needle,seen", [
+    (200, 48, 0, 152, True), (200, 48, 0, 151, False),
+    (200, 48, 5, 4, True), (200, 48, 5, 5, False),
+    (209, 64, 0, 145, True), (209, 64, 0, 144, False),
+    (330, 0, 0, 1, True), (193, 32, 40, 39, True), (50, 64, 3, 0, True)])
+@pytest.mark.parametrize("H,G,D,DV", [(4, 2, 16, 24), (8, 1, 40, 72),
+                                      (64, 2, 32, 160)])
+def test_matrix_core_attention_needles(mode, splits, T, size, keep, needle,
+                                       seen, H, G, D, DV):
+    """The same stand-out keys through the matrix-core kernel: 2, 8 and 32
+    heads per KV head, key widths that need zero padding, value widths over
+    several column blocks, portions of 1, 2 and 7 tokens, split keys."""
+    q, k, v = needle_case(T, H, G, D, DV, needle, seed=T + needle)
+    q, k, v = bf(q), bf(k), bf(v)
+    sink = torch.linspace(-1.0, 2.0, H)
+    want, p = oracle_attend(q, k, v, 0.25, size, keep, 30.0, sink)
+    assert (float(p[:, T - 1, needle].min()) > 0.9) == seen
+    got = paged(q, k, v, "cuda", sizes=_sizes(T, mode), variant_last=5,
+                dtype=torch.bfloat16, scale=0.25, window=size,
+                keep_first=keep, softcap=30.0, sink=True,
+                sink_vals=sink.cuda(), splits=splits)
+    # the output is rounded to bfloat16 once
+    assert rel_err(got.reshape(T, -1), want.reshape(T, -1)) < 6e-3
+    assert (float(got[T - 1].abs().mean()) > 20.0) == seen
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,D,DV", [(8, 136, 96), (32, 288, 256),
+                                    (2, 48, 48), (16, 584, 512)])
+@pytest.mark.parametrize("splits", [0, 4])
+def test_matrix_core_values_in_key_rows(H, D, DV, splits):
+    """Latent-attention shapes: one KV head, rows of up to 584 entries whose
+    leading entries are the values; prompt rows and single tokens."""
+    T = 75
+    g = torch.Generator().manual_seed(H + D)
+    q = bf(torch.randn(T, H, D, generator=g))
+    k = bf(torch.randn(T, 1, D, generator=g))
+    sink = torch.linspace(-1.0, 1.0, H)
+    scale = 2.0 / D ** 0.5
+    want, _ = oracle_attend(q, k, k[..., :DV], scale, 0, 0, 0.0, sink)
+    bs = 16
+    table = torch.tensor([4, 0, 3, 1, 5], dtype=torch.int32)
+    kc = torch.randn(6, 1, bs, D, generator=g)
+    pos = torch.arange(T, dtype=torch.int32)
+    slots = table[(pos // bs).long()].long() * bs + pos % bs
+    kc[(slots // bs), 0, slots % bs] = k[:, 0]
+    kc = kc.to(torch.bfloat16).cuda()
+    tq = q.reshape(T, -1).to(torch.bfloat16).cuda()
+    zero = torch.zeros(T, dtype=torch.int32, device="cuda")
+    got = ops.talk_attention(
+        tq, kc, kc, table[None].cuda(), zero, pos.cuda(), scale, H,
+        sink=True, sink_vals=sink.cuda(), vdim=DV, variant=5)
+    assert rel_err(got.float(), want.reshape(T, -1)) < 6e-3
+    # the last rows again, one token per launch row, keys split
+    got1 = ops.talk_attention(
+        tq[-9:], kc, kc, table[None].cuda(), zero[-9:], pos[-9:].cuda(),
+        scale, H, sink=True, sink_vals=sink.cuda(), vdim=DV, variant=5,
+        splits=splits)
+    assert rel_err(got1.float(), want.reshape(T, -1)[-9:]) < 6e-3
