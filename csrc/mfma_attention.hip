@@ -77,7 +77,7 @@ PS_DEV void mf_stage(unsigned short* __restrict__ dst, int pitch,
 }
 
 template <int CBW>
-__global__ __launch_bounds__(256) void mfma_attn_kernel(
+__global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     unsigned short* __restrict__ out, int ldout,
     const unsigned short* __restrict__ q, int ldq,
     const unsigned short* __restrict__ kc,
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void mfma_attn_kernel(
     const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos,
     int T_total, int H, int G, int D, int DV, int BS, float scale, int window,
-    int sink, MfOpt opt, int KS, float* __restrict__ part) {
+    int sink, MfOpt opt, int KS, float* __restrict__ part, int tpb_max) {
   extern __shared__ __align__(16) unsigned short lds16[];
   __shared__ int s_seq[32], s_pos[32];
   const int DP = (D + 15) & ~15, PK = DP + 8;
@@ -98,7 +98,9 @@ __global__ __launch_bounds__(256) void mfma_attn_kernel(
   const int row = lane & 31, hi = lane >> 5;
   const int rep = H / G;
   const int HPB = rep < 32 ? rep : 32;     // heads of a token in this group
-  const int TPB = 32 / HPB;                // tokens in this group
+  // tokens in this group; single tokens of different sequences share no
+  // keys, so a batch of them runs one token per workgroup (tpb_max = 1)
+  const int TPB = min(32 / HPB, tpb_max);
   const int hblocks = rep / HPB;
   const int g = blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
   const int ks = blockIdx.z;
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void mfma_attn_kernel(
 
   const int my_i = row / HPB;
   const int my_head = g * rep + hb * HPB + row % HPB;
-  const bool valid = my_i < ntok;
+  const bool valid = my_i < ntok;  // ntok <= TPB
   const int my_pos = valid ? s_pos[my_i] : 0;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
   const bool own_sink = sink && ks == 0;
@@ -287,23 +289,24 @@ __global__ __launch_bounds__(256) void mfma_attn_kernel(
 __global__ __launch_bounds__(256) void mfma_attn_combine_kernel(
     unsigned short* __restrict__ out, int ldout,
     const float* __restrict__ part, int H, int DV, int KS) {
-  const int t = blockIdx.x;
-  for (int c = threadIdx.x; c < H * DV; c += blockDim.x) {
-    const int h = c / DV, d = c % DV;
-    const float* rec = part + (size_t)t * KS * H * (DV + 2) + h * (DV + 2);
-    const size_t step = (size_t)H * (DV + 2);
-    float mh = PS_NEG_INF;
-    for (int s = 0; s < KS; ++s) mh = fmaxf(mh, rec[s * step]);
-    float l = 0.f, a = 0.f;
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* rec = part + ((size_t)t * KS * H + h) * (DV + 2);
+  const size_t step = (size_t)H * (DV + 2);
+  float mh = PS_NEG_INF;
+  for (int s = 0; s < KS; ++s) mh = fmaxf(mh, rec[s * step]);
+  float l = 0.f;
+  for (int s = 0; s < KS; ++s) {
+    const float ms = rec[s * step];
+    if (ms > PS_NEG_INF) l += rec[s * step + 1] * expf(ms - mh);
+  }
+  const float inv = 1.0f / l;
+  for (int d = threadIdx.x; d < DV; d += blockDim.x) {
+    float a = 0.f;
     for (int s = 0; s < KS; ++s) {
       const float ms = rec[s * step];
-      if (ms > PS_NEG_INF) {
-        const float w = expf(ms - mh);
-        l += rec[s * step + 1] * w;
-        a += rec[s * step + 2 + d] * w;
-      }
+      if (ms > PS_NEG_INF) a += rec[s * step + 2 + d] * expf(ms - mh);
     }
-    out[(size_t)t * ldout + c] = ps_f32_to_bf16(a / l);
+    out[(size_t)t * ldout + h * DV + d] = ps_f32_to_bf16(a * inv);
   }
 }
 
@@ -323,7 +326,8 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
                      int max_blocks, const void* token_seq,
                      const void* token_pos, int T_, int H, int G, int D,
                      int DV, int BS, float scale, int window, int sink,
-                     MfOpt opt, int KS, float* part, hipStream_t stream) {
+                     MfOpt opt, int KS, float* part, int tpb_max,
+                     hipStream_t stream) {
   static const size_t budget =
       mf_lds_budget((const void*)mfma_attn_kernel<CBW>);
   const int DP = (D + 15) & ~15, PK = DP + 8;
@@ -333,16 +337,18 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
   if (lds > budget) return 1;
   const int rep = H / G;
   const int HPB = rep < 32 ? rep : 32;
-  const int TPB = 32 / HPB;
+  const int TPB = 32 / HPB < tpb_max ? 32 / HPB : tpb_max;
   dim3 grid((T_ + TPB - 1) / TPB, G * (rep / HPB), KS);
   hipLaunchKernelGGL((mfma_attn_kernel<CBW>), grid, dim3(256), lds, stream,
                      (unsigned short*)out, ldout, (const unsigned short*)q,
                      ldq, (const unsigned short*)kc,
                      (const unsigned short*)vc, (const int*)block_tables,
                      max_blocks, (const int*)token_seq, (const int*)token_pos,
-                     T_, H, G, D, DV, BS, scale, window, sink, opt, KS, part);
+                     T_, H, G, D, DV, BS, scale, window, sink, opt, KS, part,
+                     tpb_max);
   if (KS > 1)
-    hipLaunchKernelGGL(mfma_attn_combine_kernel, dim3(T_), dim3(256), 0,
+    hipLaunchKernelGGL(mfma_attn_combine_kernel, dim3(T_, H),
+                       dim3(DV <= 64 ? 64 : (DV <= 128 ? 128 : 256)), 0,
                        stream, (unsigned short*)out, ldout,
                        (const float*)part, H, DV, KS);
   return 0;
@@ -357,7 +363,7 @@ extern "C" int mx_mfma_attention(
     const void* token_seq, const void* token_pos, int T_, int H, int G, int D,
     int DV, int BS, float scale, int window, int sink, int keep_first,
     float softcap, const void* sink_vals, int vrow, int v_in_k, int splits,
-    void* scratch, void* stream) {
+    void* scratch, int single_tokens, void* stream) {
   if (T_ <= 0) return 0;
   if (G < 1 || H % G) return 1;
   const int rep = H / G;
@@ -372,7 +378,7 @@ extern "C" int mx_mfma_attention(
   return mf_launch<N>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,  \
                       token_seq, token_pos, T_, H, G, D, DV, BS, scale,      \
                       window, sink, opt, KS, (float*)scratch,                \
-                      (hipStream_t)stream)
+                      single_tokens ? 1 : 32, (hipStream_t)stream)
   switch (cbw) {
     case 1: MF_GO(1);
     case 2: MF_GO(2);

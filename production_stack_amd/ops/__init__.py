@@ -679,7 +679,8 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
             int(window), int(bool(sink)), int(keep_first), _f(softcap),
             _p(sink_vals), int(VR),
             int(v_cache.data_ptr() == k_cache.data_ptr()), int(splits),
-            _p(scratch), _stream())
+            _p(scratch), int(variant == 3 or (variant == 5 and splits > 0)),
+            _stream())
         if rc == 0:
             return out
     if variant == 5:
