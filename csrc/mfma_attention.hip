@@ -13,9 +13,15 @@
 //     O^T[col, row] = V[:, col]^T . P[row, :]^T
 // so every lane's accumulator entries belong to ONE row (lane & 31): the
 // online softmax (running max, denominator, rescale) is lane-local plus one
-// exchange with lane ^ 32, and P never leaves the registers. Every wave
-// computes the full S^T of a 32-key tile and accumulates its own share of
-// the value columns (column blocks wave, wave + 4, ...).
+// exchange with lane ^ 32, and P never leaves the registers. Two ways to
+// share the work among the 4 waves:
+//   column split (ROWS = 32): every wave computes the full S^T of the 32
+//     rows and accumulates its own share of the value columns (column
+//     blocks wave, wave + 4, ...): wide values (latent attention), and
+//     single-token batches;
+//   row split (ROWS = 128): the workgroup owns 128 rows, every wave 32 of
+//     them with all value columns (at most 128): nothing is computed twice
+//     and a staged key tile serves four times as many rows.
 //
 // Scores are fp32 sums of bf16 products; the softmax is fp32; the weights
 // enter P.V as three bf16 terms (p = hi + mid + lo, each product exact,
@@ -43,40 +49,49 @@ union MfPack {
   uint4 q;
 };
 
-// Stage `rows` cache rows (keys j0 ..) of `width` elements into LDS rows of
-// `pitch` elements, zero-filled up to `wp` columns and for rows >= nk.
+// Stage the 32 cache rows whose element offsets are rowbase[0..31] (rows >=
+// nk are zero-filled) into LDS rows of `pitch` elements, `width` elements
+// each, zero-filled up to `wp` columns. The loads of a pass are all issued
+// before any is stored, so their latencies overlap.
 PS_DEV void mf_stage(unsigned short* __restrict__ dst, int pitch,
                      const unsigned short* __restrict__ cache,
-                     const int* __restrict__ table, int j0, int nk, int g,
-                     int G, int width, int wp, int BS, int RW) {
+                     const int64_t* __restrict__ rowbase, int nk, int width,
+                     int wp, bool vec) {
   const int tid = threadIdx.x, nt = blockDim.x;
-  if (width % 8 == 0 && RW % 8 == 0) {
+  if (vec) {
+    constexpr int U = 5;
     const int cpr = wp / 8;
-    for (int idx = tid; idx < 32 * cpr; idx += nt) {
-      const int row = idx / cpr, c = idx - row * cpr;
-      uint4 val = make_uint4(0, 0, 0, 0);
-      if (row < nk && c * 8 < width) {
-        const int j = j0 + row;
-        const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-        val = *(const uint4*)(cache + gb * RW + c * 8);
+    const int total = 32 * cpr;
+    for (int base = 0; base < total; base += nt * U) {
+      uint4 val[U];
+      int at[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int idx = base + u * nt + tid;
+        at[u] = -1;
+        val[u] = make_uint4(0, 0, 0, 0);
+        if (idx < total) {
+          const int row = idx / cpr, c = idx - row * cpr;
+          at[u] = row * pitch + c * 8;
+          if (row < nk && c * 8 < width)
+            val[u] = *(const uint4*)(cache + rowbase[row] + c * 8);
+        }
       }
-      *(uint4*)(dst + row * pitch + c * 8) = val;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (at[u] >= 0) *(uint4*)(dst + at[u]) = val[u];
     }
   } else {
     for (int idx = tid; idx < 32 * wp; idx += nt) {
       const int row = idx / wp, c = idx - row * wp;
       unsigned short val = 0;
-      if (row < nk && c < width) {
-        const int j = j0 + row;
-        const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-        val = cache[gb * RW + c];
-      }
+      if (row < nk && c < width) val = cache[rowbase[row] + c];
       dst[row * pitch + c] = val;
     }
   }
 }
 
-template <int CBW>
+template <int CBW, int ROWS>
 __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     unsigned short* __restrict__ out, int ldout,
     const unsigned short* __restrict__ q, int ldq,
@@ -87,20 +102,23 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     int T_total, int H, int G, int D, int DV, int BS, float scale, int window,
     int sink, MfOpt opt, int KS, float* __restrict__ part, int tpb_max) {
   extern __shared__ __align__(16) unsigned short lds16[];
-  __shared__ int s_seq[32], s_pos[32];
+  __shared__ int s_seq[ROWS], s_pos[ROWS];
+  __shared__ int64_t s_kbase[32], s_vbase[32];
   const int DP = (D + 15) & ~15, PK = DP + 8;
   const int DVP = (DV + 31) & ~31, PV = opt.v_in_k ? PK : DVP + 8;
-  unsigned short* sQ = lds16;              // [32][PK]
-  unsigned short* sK = sQ + 32 * PK;       // [32][PK]
+  unsigned short* sQ = lds16;              // [ROWS][PK]
+  unsigned short* sK = sQ + ROWS * PK;     // [32][PK]
   unsigned short* sV = opt.v_in_k ? sK : sK + 32 * PK;   // [32][PV]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int row = lane & 31, hi = lane >> 5;
+  // this wave's row of the workgroup
+  const int grow = (ROWS == 32 ? 0 : wave * 32) + row;
   const int rep = H / G;
   const int HPB = rep < 32 ? rep : 32;     // heads of a token in this group
   // tokens in this group; single tokens of different sequences share no
   // keys, so a batch of them runs one token per workgroup (tpb_max = 1)
-  const int TPB = min(32 / HPB, tpb_max);
+  const int TPB = min(ROWS / HPB, tpb_max);
   const int hblocks = rep / HPB;
   const int g = blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
   const int ks = blockIdx.z;
@@ -112,17 +130,31 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     s_pos[c] = token_pos[tok0 + c];
   }
   // queries of the 32 rows, zero-padded
-  for (int idx = tid; idx < 32 * DP; idx += blockDim.x) {
-    const int r = idx / DP, d = idx - r * DP;
-    const int i = r / HPB, head = g * rep + hb * HPB + r % HPB;
-    unsigned short val = 0;
-    if (i < ntok && d < D) val = q[(size_t)(tok0 + i) * ldq + head * D + d];
-    sQ[r * PK + d] = val;
+  const bool kvec = D % 8 == 0;
+  const bool vvec = DV % 8 == 0 && opt.vr % 8 == 0;
+  if (kvec && ldq % 8 == 0 && ((size_t)q & 15) == 0) {
+    const int cpr = DP / 8;
+    for (int idx = tid; idx < ROWS * cpr; idx += blockDim.x) {
+      const int r = idx / cpr, c = idx - r * cpr;
+      const int i = r / HPB, head = g * rep + hb * HPB + r % HPB;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (i < ntok && c * 8 < D)
+        val = *(const uint4*)(q + (size_t)(tok0 + i) * ldq + head * D + c * 8);
+      *(uint4*)(sQ + r * PK + c * 8) = val;
+    }
+  } else {
+    for (int idx = tid; idx < ROWS * DP; idx += blockDim.x) {
+      const int r = idx / DP, d = idx - r * DP;
+      const int i = r / HPB, head = g * rep + hb * HPB + r % HPB;
+      unsigned short val = 0;
+      if (i < ntok && d < D) val = q[(size_t)(tok0 + i) * ldq + head * D + d];
+      sQ[r * PK + d] = val;
+    }
   }
   __syncthreads();
 
-  const int my_i = row / HPB;
-  const int my_head = g * rep + hb * HPB + row % HPB;
+  const int my_i = grow / HPB;
+  const int my_head = g * rep + hb * HPB + grow % HPB;
   const bool valid = my_i < ntok;  // ntok <= TPB
   const int my_pos = valid ? s_pos[my_i] : 0;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
@@ -155,16 +187,22 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
         if (tile_no % KS != ks) continue;
         const int nk = min(32, rb + 1 - j0);
         __syncthreads();  // the previous tile is fully consumed
-        mf_stage(sK, PK, kc, table, j0, nk, g, G, D, DP, BS, D);
-        if (!opt.v_in_k)
-          mf_stage(sV, PV, vc, table, j0, nk, g, G, DV, DVP, BS, opt.vr);
+        if (tid < nk) {
+          const int j = j0 + tid;
+          const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+          s_kbase[tid] = gb * D;
+          s_vbase[tid] = gb * opt.vr;
+        }
+        __syncthreads();
+        mf_stage(sK, PK, kc, s_kbase, nk, D, DP, kvec);
+        if (!opt.v_in_k) mf_stage(sV, PV, vc, s_vbase, nk, DV, DVP, vvec);
         __syncthreads();
 
         mf_f32x16 st;
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[r] = 0.f;
         const unsigned short* ka = sK + row * PK + 8 * hi;
-        const unsigned short* qb = sQ + row * PK + 8 * hi;
+        const unsigned short* qb = sQ + grow * PK + 8 * hi;
         for (int k0 = 0; k0 < DP; k0 += 16) {
           const mf_bf16x8 a = *(const mf_bf16x8*)(ka + k0);
           const mf_bf16x8 b = *(const mf_bf16x8*)(qb + k0);
@@ -227,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
           }
 #pragma unroll
           for (int c = 0; c < CBW; ++c) {
-            const int cb = wave + 4 * c;
+            const int cb = ROWS == 32 ? wave + 4 * c : c;
             if (cb * 32 < DV) {
               MfPack a;
               const unsigned short* vp = sV + cb * 32 + row;
@@ -257,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     unsigned short* o = out + (size_t)(tok0 + my_i) * ldout + my_head * DV;
 #pragma unroll
     for (int c = 0; c < CBW; ++c) {
-      const int cb = wave + 4 * c;
+      const int cb = ROWS == 32 ? wave + 4 * c : c;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int col = cb * 32 + (r & 3) + 8 * (r >> 2) + 4 * hi;
@@ -268,13 +306,13 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     // partial record per (token, share, head): max, denominator, DV sums
     float* rec = part + (((size_t)(tok0 + my_i) * KS + ks) * H + my_head) *
                             (size_t)(DV + 2);
-    if (hi == 0 && wave == 0) {
+    if (hi == 0 && (wave == 0 || ROWS != 32)) {
       rec[0] = m;
       rec[1] = l;
     }
 #pragma unroll
     for (int c = 0; c < CBW; ++c) {
-      const int cb = wave + 4 * c;
+      const int cb = ROWS == 32 ? wave + 4 * c : c;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int col = cb * 32 + (r & 3) + 8 * (r >> 2) + 4 * hi;
@@ -320,7 +358,7 @@ static size_t mf_lds_budget(const void* fn) {
   return 64 * 1024;
 }
 
-template <int CBW>
+template <int CBW, int ROWS>
 static int mf_launch(void* out, int ldout, const void* q, int ldq,
                      const void* kc, const void* vc, const void* block_tables,
                      int max_blocks, const void* token_seq,
@@ -329,17 +367,18 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
                      MfOpt opt, int KS, float* part, int tpb_max,
                      hipStream_t stream) {
   static const size_t budget =
-      mf_lds_budget((const void*)mfma_attn_kernel<CBW>);
+      mf_lds_budget((const void*)mfma_attn_kernel<CBW, ROWS>);
   const int DP = (D + 15) & ~15, PK = DP + 8;
   const int DVP = (DV + 31) & ~31;
-  const size_t lds =
-      ((size_t)64 * PK + (opt.v_in_k ? 0 : (size_t)32 * (DVP + 8))) * 2;
+  const size_t lds = ((size_t)(ROWS + 32) * PK +
+                      (opt.v_in_k ? 0 : (size_t)32 * (DVP + 8))) * 2;
   if (lds > budget) return 1;
   const int rep = H / G;
   const int HPB = rep < 32 ? rep : 32;
-  const int TPB = 32 / HPB < tpb_max ? 32 / HPB : tpb_max;
+  const int TPB = ROWS / HPB < tpb_max ? ROWS / HPB : tpb_max;
   dim3 grid((T_ + TPB - 1) / TPB, G * (rep / HPB), KS);
-  hipLaunchKernelGGL((mfma_attn_kernel<CBW>), grid, dim3(256), lds, stream,
+  hipLaunchKernelGGL((mfma_attn_kernel<CBW, ROWS>), grid, dim3(256), lds,
+                     stream,
                      (unsigned short*)out, ldout, (const unsigned short*)q,
                      ldq, (const unsigned short*)kc,
                      (const unsigned short*)vc, (const int*)block_tables,
@@ -356,14 +395,17 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
 
 // Returns 0 when launched, 1 when the shape is outside this kernel (the
 // caller then takes the vector kernels): heads per KV head must divide 32
-// or be a multiple of 32, at most 512 value columns.
+// or be a multiple of 32, at most 512 value columns. mode 0: prompt
+// portions (row split for large batches of narrow values, else column
+// split), 1: single tokens of different sequences (one token per
+// workgroup), 2: row split whatever the batch size.
 extern "C" int mx_mfma_attention(
     void* out, int ldout, const void* q, int ldq, const void* kc,
     const void* vc, const void* block_tables, int max_blocks,
     const void* token_seq, const void* token_pos, int T_, int H, int G, int D,
     int DV, int BS, float scale, int window, int sink, int keep_first,
     float softcap, const void* sink_vals, int vrow, int v_in_k, int splits,
-    void* scratch, int single_tokens, void* stream) {
+    void* scratch, int mode, void* stream) {
   if (T_ <= 0) return 0;
   if (G < 1 || H % G) return 1;
   const int rep = H / G;
@@ -375,10 +417,20 @@ extern "C" int mx_mfma_attention(
   int KS = splits > 1 && scratch != nullptr ? splits : 1;
   const int cbw = ((DV + 31) / 32 + 3) / 4;
 #define MF_GO(N)                                                             \
-  return mf_launch<N>(out, ldout, q, ldq, kc, vc, block_tables, max_blocks,  \
-                      token_seq, token_pos, T_, H, G, D, DV, BS, scale,      \
-                      window, sink, opt, KS, (float*)scratch,                \
-                      single_tokens ? 1 : 32, (hipStream_t)stream)
+  return mf_launch<N, 32>(out, ldout, q, ldq, kc, vc, block_tables,          \
+                          max_blocks, token_seq, token_pos, T_, H, G, D, DV, \
+                          BS, scale, window, sink, opt, KS, (float*)scratch, \
+                          mode == 1 ? 1 : 128, (hipStream_t)stream)
+  // prompt portions with at most 128 value columns: row split (unless the
+  // batch is too small to fill the chip with 128-row workgroups)
+  if (DV <= 128 && rep <= 32 &&
+      (mode == 2 || (mode == 0 && (long)T_ * H >= 128L * 512))) {
+    const int rc = mf_launch<4, 128>(
+        out, ldout, q, ldq, kc, vc, block_tables, max_blocks, token_seq,
+        token_pos, T_, H, G, D, DV, BS, scale, window, sink, opt, KS,
+        (float*)scratch, 128, (hipStream_t)stream);
+    if (rc == 0) return 0;
+  }
   switch (cbw) {
     case 1: MF_GO(1);
     case 2: MF_GO(2);

@@ -624,7 +624,7 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     both falling back to the plain one-workgroup-per-token kernel; 1 / 2 /
     4 force plain / tiled / split-key. bfloat16 batches without head mix
     and aligned chunks take the matrix-core kernel instead when the shape
-    fits it (variants 0 and 3; 5 insists on it).
+    fits it (variants 0 and 3; 5 insists on it, 6 on its 128-row form).
     Returns [T, H*DV]."""
     NB, G, BS, D = k_cache.shape
     VR = v_cache.shape[3]
@@ -660,18 +660,21 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     # workgroup per token, each token's keys are shared out over several
     # workgroups whose partial softmax records are merged afterwards
     scratch = None
-    if variant not in (3, 4, 5):
+    if variant not in (3, 4, 5, 6):
         splits = 1
     elif splits <= 0:
         splits = (max(1, min(8, 512 // T))
-                  if T < 256 and variant != 5 else 1)
+                  if T < 256 and variant not in (5, 6) else 1)
     if splits > 1:
         scratch = torch.empty((T, splits, H, DV + 2),
                               dtype=torch.float32, device=q.device)
     # bf16 without head mix / aligned chunks: the matrix-core kernel, where
     # the shape fits it (variant 5 insists on it)
-    if (variant in (0, 3, 5) and q.dtype == torch.bfloat16 and talk is None
-            and chunk == 0):
+    if (variant in (0, 3, 5, 6) and q.dtype == torch.bfloat16
+            and talk is None and chunk == 0):
+        # 0: prompt portions, 1: single tokens, 2: 128-row workgroups
+        mode = (2 if variant == 6 else
+                int(variant == 3 or (variant == 5 and splits > 0)))
         rc = _mx().mx_mfma_attention(
             _p(out), _rows(out, "out"), _p(q), _rows(q, "q"), _p(k_cache),
             _p(v_cache), _p(block_tables), block_tables.shape[1],
@@ -679,11 +682,10 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
             int(window), int(bool(sink)), int(keep_first), _f(softcap),
             _p(sink_vals), int(VR),
             int(v_cache.data_ptr() == k_cache.data_ptr()), int(splits),
-            _p(scratch), int(variant == 3 or (variant == 5 and splits > 0)),
-            _stream())
+            _p(scratch), mode, _stream())
         if rc == 0:
             return out
-    if variant == 5:
+    if variant in (5, 6):
         raise RuntimeError(
             "talk_attention: shape or dtype outside the matrix-core kernel")
     rc = _mx().mx_talk_attention(
