@@ -69,22 +69,92 @@ __global__ __launch_bounds__(MAXT) void gated_delta_kernel(
     S[r] = (col && i < D && p0 != 0) ? Sg[(size_t)i * DV + j] : 0.f;
   }
 
+  // The inputs of tile t+1 are fetched into registers before tile t is
+  // swept, so their global-memory latency hides behind the sweep. A thread
+  // prepares elements tid + e * blockDim of a tile (token-major, DKP per
+  // token); the first NE of them go through the registers, any beyond that
+  // (few columns on a tall state) are loaded when the tile is committed.
+  // (a 1024-thread launch has 128 registers a lane: no room for them).
+  // Fetching ahead pays for launches of up to 256 threads; wider ones
+  // (measured: 512 threads on 128 x 128 states) are bound by the sweep's
+  // LDS reads and run faster when a tile's inputs are fetched at its start.
+  constexpr bool AHEAD = MAXT <= 256;
+  constexpr int NE = AHEAD ? 8 : 0;
+  constexpr int NEA = NE > 0 ? NE : 1;
+  float pk[NEA], pq[NEA], pz[NEA], pdt[NEA];
+  constexpr int TA = AHEAD ? TILE : 1;
+  float vnext[TA], gnext[TA];
+  float bnext = 0.f;
+#pragma unroll
+  for (int e = 0; e < NE; ++e) {
+    const int i = (threadIdx.x + e * blockDim.x) % DKP;
+    pdt[e] = i < D ? dt_bias[hz + i] : 0.f;
+  }
+  auto prefetch = [&](int tb) {
+    const int nt = min(TILE, n - tb);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      const int idx = threadIdx.x + e * blockDim.x;
+      const int tt = idx / DKP, i = idx % DKP;
+      pk[e] = pq[e] = pz[e] = 0.f;
+      if (idx < nt * DKP && i < D) {
+        const size_t row = (size_t)(t0 + tb + tt);
+        pk[e] = MxElem<T>::ld(k + row * ldk + hk + i);
+        pq[e] = MxElem<T>::ld(q + row * ldq + hk + i);
+        pz[e] = MxElem<T>::ld(zdec + row * ldzd + hz + i);
+      }
+    }
+#pragma unroll
+    for (int tt = 0; tt < TA; ++tt) {
+      const size_t row = (size_t)(t0 + tb + min(tt, nt - 1));
+      vnext[tt] = col ? MxElem<T>::ld(v + row * ldv + hv + j) : 0.f;
+      gnext[tt] = col ? MxElem<T>::ld(zgate + row * ldzg + hv + j) : 0.f;
+    }
+    if (threadIdx.x < nt)
+      bnext = MxElem<T>::ld(beta + (size_t)(t0 + tb + threadIdx.x) * ldb + hd);
+  };
+  if (AHEAD) prefetch(0);
+
   for (int tb = 0; tb < n; tb += TILE) {
     const int nt = min(TILE, n - tb);
     __syncthreads();  // previous tile's LDS reads are done
     float vreg[TILE], greg[TILE];
+    if constexpr (AHEAD) {
 #pragma unroll
-    for (int tt = 0; tt < TILE; ++tt) {
-      const size_t row = (size_t)(t0 + tb + min(tt, nt - 1));
-      vreg[tt] = col ? MxElem<T>::ld(v + row * ldv + hv + j) : 0.f;
-      greg[tt] = col ? MxElem<T>::ld(zgate + row * ldzg + hv + j) : 0.f;
+      for (int tt = 0; tt < TILE; ++tt) {
+        vreg[tt] = vnext[tt];
+        greg[tt] = gnext[tt];
+      }
+      if (threadIdx.x < nt) sbeta[threadIdx.x] = mx_sigmoid(bnext);
+    } else {
+      // this tile's value and gate entries of column j: issued together,
+      // up front, so their latency hides behind the preparation
+#pragma unroll
+      for (int tt = 0; tt < TILE; ++tt) {
+        const size_t row = (size_t)(t0 + tb + min(tt, nt - 1));
+        vreg[tt] = col ? MxElem<T>::ld(v + row * ldv + hv + j) : 0.f;
+        greg[tt] = col ? MxElem<T>::ld(zgate + row * ldzg + hv + j) : 0.f;
+      }
+      if (threadIdx.x < nt)
+        sbeta[threadIdx.x] = mx_sigmoid(MxElem<T>::ld(
+            beta + (size_t)(t0 + tb + threadIdx.x) * ldb + hd));
     }
-    if (threadIdx.x < nt)
-      sbeta[threadIdx.x] = mx_sigmoid(MxElem<T>::ld(
-          beta + (size_t)(t0 + tb + threadIdx.x) * ldb + hd));
-    for (int idx = threadIdx.x; idx < nt * DKP; idx += blockDim.x) {
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      const int idx = threadIdx.x + e * blockDim.x;
+      if (idx < nt * DKP) {
+        const int tt = idx / DKP, i = idx % DKP;
+        // row i is kept at (i % P) * RP + i / P: a lane's rows are
+        // contiguous
+        const int at = tt * TP + (i % P) * RP + i / P;
+        sk[at] = pk[e];
+        sq[at] = pq[e];
+        sg[at] = i < D ? expf(-rate * mx_softplus(pz[e] + pdt[e])) : 0.f;
+      }
+    }
+    for (int idx = threadIdx.x + NE * blockDim.x; idx < nt * DKP;
+         idx += blockDim.x) {
       const int tt = idx / DKP, i = idx % DKP;
-      // row i is kept at (i % P) * RP + i / P: a lane's rows are contiguous
       const int at = tt * TP + (i % P) * RP + i / P;
       float kv = 0.f, qv = 0.f, gv = 0.f;
       if (i < D) {
@@ -98,6 +168,7 @@ __global__ __launch_bounds__(MAXT) void gated_delta_kernel(
       sq[at] = qv;
       sg[at] = gv;
     }
+    if (AHEAD && tb + TILE < n) prefetch(tb + TILE);
     __syncthreads();
     for (int tt = wave; tt < nt; tt += nw) {
       float sk2 = 0.f, sq2 = 0.f;
@@ -221,10 +292,12 @@ static int launch_gated_delta(GD_ARGS) {
                      (const float*)dt_bias, (const float*)normw,             \
                      (float*)state, (const int*)seq_rows, H, G, D, DV, eps,  \
                      qscale)
-  // tall states with up to 128 columns get the registers of a 512-thread
-  // launch (a lane's rows stay out of scratch memory)
-  if (DKP >= 96 && threads <= 512) {
-    GD_LAUNCH((DKP >= 96 ? 512 : 1024));
+  // the launch bound follows the thread count, so small launches get the
+  // registers for the prefetched tile and a lane's rows stay out of scratch
+  if (threads <= 256) {
+    GD_LAUNCH(256);
+  } else if (threads <= 512) {
+    GD_LAUNCH(512);
   } else {
     GD_LAUNCH(1024);
   }
