@@ -8,7 +8,10 @@ hipGraph on ROCm) against static input buffers and replayed each step.
 
 Padding rows are made harmless by: slot_mapping = -1 (KV append skips),
 seq_len = 1 with block_table row 0 (reads one garbage block, output row is
-discarded), token id 0, position 0.
+discarded), token id 0, position 0. Families with per-sequence recurrent
+state (needs_seq_meta) also get static whole-batch metadata: every row is a
+one-token segment [row, 1, position, state slot]; padding rows use a spare
+state slot that no sequence owns.
 """
 
 from __future__ import annotations
@@ -34,6 +37,7 @@ class DecodeGraphRunner:
         max_batch: int,
         max_blocks_per_seq: int,
         device: torch.device,
+        pad_state_slot: int = 0,
     ) -> None:
         self.model = model
         self.kv_caches = kv_caches
@@ -67,6 +71,17 @@ class DecodeGraphRunner:
         self.h_lora_idx = torch.full((B,), -1, dtype=torch.int32,
                                      pin_memory=True)
         self.use_lora = getattr(model, "lora_slots", None) is not None
+        # whole-batch sequence metadata for hybrid recurrent/attention stacks
+        self.seq_meta = bool(getattr(model, "needs_seq_meta", False))
+        self.pad_state_slot = pad_state_slot
+        if self.seq_meta:
+            rows = np.zeros((B, 4), dtype=np.int32)
+            rows[:, 0] = np.arange(B)
+            rows[:, 1] = 1
+            rows[:, 3] = pad_state_slot
+            self.h_seq_rows = torch.from_numpy(rows.copy()).pin_memory()
+            self.seq_rows = torch.from_numpy(rows).to(dev)
+            self.token_seq = torch.arange(B, dtype=torch.int32, device=dev)
 
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self.logits: Dict[int, torch.Tensor] = {}
@@ -84,6 +99,9 @@ class DecodeGraphRunner:
             decode_seq_lens=self.seq_lens[:b],
             decode_block_tables=self.block_tables[:b],
             lora_idx=self.lora_idx[:b] if self.use_lora else None,
+            **(dict(block_tables=self.block_tables[:b],
+                    token_seq=self.token_seq[:b],
+                    seq_rows=self.seq_rows[:b]) if self.seq_meta else {}),
         )
 
     @torch.no_grad()
@@ -135,6 +153,7 @@ class DecodeGraphRunner:
         block_tables: List[List[int]],
         lora_idx: Optional[np.ndarray] = None,
         prev_fill=None,  # (rows, src_rows, prev_sampled_dev) async gather
+        state_slots: Optional[np.ndarray] = None,
     ) -> torch.Tensor:
         n = len(tokens)
         b = self.bucket_for(n)
@@ -152,6 +171,13 @@ class DecodeGraphRunner:
         for i, bt in enumerate(block_tables):
             hbt[i, : len(bt)] = bt
         hbt[n:b, 0] = 0
+        if self.seq_meta:
+            hsr = self.h_seq_rows.numpy()
+            hsr[:n, 2] = positions
+            hsr[:n, 3] = state_slots
+            hsr[n:b, 2] = 0
+            hsr[n:b, 3] = self.pad_state_slot
+            self.seq_rows[:b].copy_(self.h_seq_rows[:b], non_blocking=True)
         if self.use_lora:
             if lora_idx is None:
                 self.h_lora_idx[:b] = -1

@@ -157,7 +157,9 @@ class ModelRunner:
                     "this model family keeps its KV cache in the serving "
                     "dtype (no fp8 KV)")
             dt = self.model.dtype
-            slots = max(self.num_state_slots, 1)
+            # one spare slot past the sequences': padding rows of captured
+            # decode graphs park their state there
+            slots = self.num_state_slots + 1
 
             def alloc(desc):
                 kind = desc[0]
@@ -247,8 +249,9 @@ class ModelRunner:
         from production_stack_amd.engine.graph_runner import DecodeGraphRunner
         from production_stack_amd.ops import gemm_policy
 
-        # fp8-quantized GEMMs run through scaled_mm: nothing to autotune
-        if self.config.quantization != "fp8":
+        # fp8-quantized GEMMs run through scaled_mm: nothing to autotune;
+        # heterogeneous stacks were tuned above over all their shapes
+        if self.config.quantization != "fp8" and not self.hybrid:
             try:
                 layer0 = self.model.layers[0]
                 weights = [
@@ -271,7 +274,8 @@ class ModelRunner:
         ) // self.config.cache.block_size
         try:
             runner = DecodeGraphRunner(
-                self.model, self.kv_caches, max_batch, max_blocks, self.device
+                self.model, self.kv_caches, max_batch, max_blocks,
+                self.device, pad_state_slot=self.num_state_slots,
             )
             runner.capture_all()
             self.graphs = runner
@@ -548,6 +552,9 @@ class ModelRunner:
         lora_idx = None
         if self.lora_slots is not None:
             lora_idx = np.full(n, -1, dtype=np.int32)
+        state_slots = None
+        if self.graphs.seq_meta:
+            state_slots = np.zeros(n, dtype=np.int32)
         ph_rows: List[int] = []
         ph_src: List[int] = []
         for i, ss in enumerate(scheduled):
@@ -571,6 +578,15 @@ class ModelRunner:
             seq_lens[i] = pos + 1
             tables.append(seq.block_table)
             seqs.append(seq)
+            if state_slots is not None:
+                slot = seq.state_slot
+                if self.num_state_slots and not (
+                        slot is not None
+                        and 0 <= slot < self.num_state_slots):
+                    raise RuntimeError(
+                        f"sequence {seq.request_id} has no valid "
+                        "recurrent-state slot")
+                state_slots[i] = slot or 0
             if lora_idx is not None and seq.lora_name:
                 lora_idx[i] = self.lora_slots.slot_by_name.get(
                     seq.lora_name, -1
@@ -579,7 +595,7 @@ class ModelRunner:
         if ph_rows:
             prev_fill = (ph_rows, ph_src, self._prev_tokens_dev)
         logits = self.graphs.run(tokens, positions, slots, seq_lens, tables,
-                                 lora_idx, prev_fill)
+                                 lora_idx, prev_fill, state_slots)
         if defer_sample:
             return logits, seqs
         sampled = self.sample(logits, seqs)

@@ -185,7 +185,8 @@ class DerusunLayer(nn.Module):
 class DerusunForCausalLM(nn.Module):
     # per-step metadata this family needs from the runner
     needs_seq_meta = True
-    supports_decode_graph = False
+    # no data-dependent control flow: single-token steps replay a hipGraph
+    supports_decode_graph = True
 
     def __init__(self, cfg: ModelConfig, tp: int = 1, pp_rank: int = 0,
                  pp_size: int = 1, dtype: torch.dtype = torch.bfloat16
