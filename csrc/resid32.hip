@@ -31,28 +31,6 @@ PS_DEV void mx_group_inv(const float* __restrict__ xr, int W, int groups,
   __syncthreads();
 }
 
-// Rows of up to MX_ROW_REGS * 256 entries are held in registers (entry
-// tid + 256 k in slot k), so global memory is read once.
-#define MX_ROW_REGS 32
-
-// 1/rms per group of a row held in registers; sinv[groups] in LDS. Ends
-// with a barrier.
-PS_DEV void mx_group_inv_regs(const float* v, int W, int groups, float eps,
-                              float* sinv, float* red) {
-  const int gw = W / groups;
-  for (int g = 0; g < groups; ++g) {
-    float ss = 0.f;
-#pragma unroll
-    for (int k = 0; k < MX_ROW_REGS; ++k) {
-      const int c = threadIdx.x + 256 * k;
-      if (c < W && c / gw == g) ss += v[k] * v[k];
-    }
-    ss = mx_block_sum(ss, red);
-    if (threadIdx.x == 0) sinv[g] = 1.0f / sqrtf(ss / (float)gw + eps);
-  }
-  __syncthreads();
-}
-
 // xo[t] = xi[t] + d0[t] + d1[t] (each optional; xo may be xi),
 // h[t] = xo[t] / rms(part of xo[t]) * w, one rms per group of W / groups.
 template <typename T>
@@ -65,32 +43,6 @@ __global__ __launch_bounds__(256) void add_group_norm32_kernel(
   const int t = blockIdx.x;
   float* xr = xo + (size_t)t * W;
   const float* xs = xi + (size_t)t * W;
-  const int gw = W / groups;
-  if (W <= MX_ROW_REGS * 256) {
-    float v[MX_ROW_REGS];
-#pragma unroll
-    for (int k = 0; k < MX_ROW_REGS; ++k) {
-      const int c = threadIdx.x + 256 * k;
-      v[k] = 0.f;
-      if (c < W) {
-        v[k] = xs[c];
-        if (d0 != nullptr) {
-          float d = MxElem<T>::ld(d0 + (size_t)t * ld0 + c);
-          if (d1 != nullptr) d += MxElem<T>::ld(d1 + (size_t)t * ld1 + c);
-          v[k] += d;
-        }
-        if (d0 != nullptr || xo != xi) xr[c] = v[k];
-      }
-    }
-    mx_group_inv_regs(v, W, groups, eps, sinv, red);
-#pragma unroll
-    for (int k = 0; k < MX_ROW_REGS; ++k) {
-      const int c = threadIdx.x + 256 * k;
-      if (c < W)
-        MxElem<T>::st(h + (size_t)t * W + c, v[k] * sinv[c / gw] * w[c]);
-    }
-    return;
-  }
   if (d0 != nullptr || xo != xi) {
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
       float v = xs[c];
@@ -104,6 +56,7 @@ __global__ __launch_bounds__(256) void add_group_norm32_kernel(
     __syncthreads();  // the sums below read other threads' entries
   }
   mx_group_inv(xr, W, groups, eps, sinv, red);
+  const int gw = W / groups;
   for (int c = threadIdx.x; c < W; c += blockDim.x)
     MxElem<T>::st(h + (size_t)t * W + c, xr[c] * sinv[c / gw] * w[c]);
 }
@@ -131,61 +84,11 @@ __global__ __launch_bounds__(256) void group_norm_shift_kernel(
   const float* xr = x + (size_t)t * W;
   const float* xp = x + (size_t)(first ? t : t - 1) * W;
   const float* xl = x + (size_t)last * W;
-  const int gw = W / groups;
-  float* st = state + (size_t)slot * W;
-  if (W <= (MX_ROW_REGS / 2) * 256) {
-    // own row and the other row needed (predecessor, or for a segment's
-    // first row its last row) both stay in registers
-    constexpr int NR = MX_ROW_REGS / 2;
-    const bool other = !first || n > 1;
-    const float* xq = first ? xl : xp;
-    float a[NR], b[NR];
-#pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      const int c = threadIdx.x + 256 * k;
-      a[k] = c < W ? xr[c] : 0.f;
-      b[k] = (other && c < W) ? xq[c] : 0.f;
-    }
-    for (int g = 0; g < groups; ++g) {
-      float sa = 0.f, sb = 0.f;
-#pragma unroll
-      for (int k = 0; k < NR; ++k) {
-        const int c = threadIdx.x + 256 * k;
-        if (c < W && c / gw == g) {
-          sa += a[k] * a[k];
-          sb += b[k] * b[k];
-        }
-      }
-      sa = mx_block_sum(sa, red);
-      sb = mx_block_sum(sb, red);
-      if (threadIdx.x == 0) {
-        sinv[0][g] = 1.0f / sqrtf(sa / (float)gw + eps);
-        sinv[1][g] = 1.0f / sqrtf(sb / (float)gw + eps);
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      const int c = threadIdx.x + 256 * k;
-      if (c < W) {
-        const int g = c / gw;
-        const float hn = a[k] * sinv[0][g] * w[c];
-        const float ho = b[k] * sinv[1][g] * w[c];
-        float prev;
-        if (!first) {
-          prev = ho;
-        } else {
-          prev = p0 > 0 ? st[c] : 0.f;
-          st[c] = n > 1 ? ho : hn;
-        }
-        MxElem<T>::st(h + (size_t)t * W + c, hn + (prev - hn) * shift[c]);
-      }
-    }
-    return;
-  }
   mx_group_inv(xr, W, groups, eps, sinv[0], red);
   if (!first) mx_group_inv(xp, W, groups, eps, sinv[1], red);
   if (first && n > 1) mx_group_inv(xl, W, groups, eps, sinv[2], red);
+  const int gw = W / groups;
+  float* st = state + (size_t)slot * W;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const int g = c / gw;
     const float hn = xr[c] * sinv[0][g] * w[c];

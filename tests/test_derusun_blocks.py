@@ -585,25 +585,28 @@ def bf(x):
     return x.to(torch.bfloat16).float()
 
 
+MC_SHAPES = [(4, 2, 16, 24), (8, 1, 40, 72), (64, 2, 32, 160)]
+MC_MODES = [((None,), 0, 5), ((0, 1), 0, 5), ((0, 1), 3, 5), ((0, 2), 0, 5),
+            ((0, 7), 0, 5), ((None,), 0, 6), ((0, 7), 0, 6),
+            ((0, 150), 0, 6)]
+# the 128-row form (variant 6) holds at most 128 value columns
+MC_CASES = [(m, sh) for m in MC_MODES for sh in MC_SHAPES
+            if not (m[2] == 6 and sh[3] > 128)]
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("mode,splits,variant", [
-    ((None,), 0, 5), ((0, 1), 0, 5), ((0, 1), 3, 5), ((0, 2), 0, 5),
-    ((0, 7), 0, 5), ((None,), 0, 6), ((0, 7), 0, 6), ((0, 150), 0, 6)])
 @pytest.mark.parametrize("T,size,keep,needle,seen", [
     (200, 48, 0, 152, True), (200, 48, 0, 151, False),
     (200, 48, 5, 4, True), (200, 48, 5, 5, False),
     (209, 64, 0, 145, True), (209, 64, 0, 144, False),
     (330, 0, 0, 1, True), (193, 32, 40, 39, True), (50, 64, 3, 0, True)])
-@pytest.mark.parametrize("H,G,D,DV", [(4, 2, 16, 24), (8, 1, 40, 72),
-                                      (64, 2, 32, 160)])
-def test_matrix_core_attention_needles(mode, splits, variant, T, size, keep,
-                                       needle, seen, H, G, D, DV):
+@pytest.mark.parametrize("case", MC_CASES)
+def test_matrix_core_attention_needles(case, T, size, keep, needle, seen):
     """The same stand-out keys through the matrix-core kernel: 2, 8 and 32
     heads per KV head, key widths that need zero padding, value widths over
     several column blocks, portions of 1, 2 and 7 tokens, split keys; the
     128-row form (variant 6) on whole prompts and portions."""
-    if variant == 6 and DV > 128:
-        pytest.skip("the 128-row form holds at most 128 value columns")
+    (mode, splits, variant), (H, G, D, DV) = case
     q, k, v = needle_case(T, H, G, D, DV, needle, seed=T + needle)
     q, k, v = bf(q), bf(k), bf(v)
     sink = torch.linspace(-1.0, 2.0, H)
