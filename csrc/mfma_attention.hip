@@ -43,6 +43,18 @@ struct MfOpt {
   int v_in_k;    // values are read from the key rows
 };
 
+// The softmax arithmetic of a tile is repeated by every wave that owns
+// columns of the same rows, and a wave64 instruction takes four cycles, so
+// the exponential and the cap use the hardware exponential (fp32, a few
+// ulp) instead of the library's range-checked forms:
+// tanh(x) = 1 - 2 / (exp(2x) + 1).
+PS_DEV float mf_exp(float x) { return __expf(x); }
+
+PS_DEV float mf_cap(float sc, float cap, float inv_cap2) {
+  const float e = __expf(sc * inv_cap2);  // exp(2 sc / cap); inf is fine
+  return cap * (1.0f - __fdividef(2.0f, e + 1.0f));
+}
+
 union MfPack {
   mf_bf16x8 v;
   unsigned short u[8];
@@ -158,6 +170,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
   const bool valid = my_i < ntok;  // ntok <= TPB
   const int my_pos = valid ? s_pos[my_i] : 0;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const float inv_cap2 = opt.softcap > 0.f ? 2.0f / opt.softcap : 0.f;
   const bool own_sink = sink && ks == 0;
   float m = own_sink ? (opt.sink_vals ? opt.sink_vals[my_head] : 0.f)
                      : PS_NEG_INF;
@@ -216,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
           const int kk = (r & 3) + 8 * (r >> 2) + 4 * hi;
           const int j = j0 + kk;
           float sc = st[r] * scale;
-          if (opt.softcap > 0.f) sc = opt.softcap * tanhf(sc / opt.softcap);
+          if (opt.softcap > 0.f) sc = mf_cap(sc, opt.softcap, inv_cap2);
           const bool vis = mine && kk < nk && j <= my_pos &&
                            (j >= my_lo || j < opt.keep_first);
           sc = vis ? sc : PS_NEG_INF;
@@ -227,11 +240,11 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
         const float mnew = fmaxf(m, mx);
         float alpha = 1.f;
         if (mnew > PS_NEG_INF) {
-          alpha = expf(m - mnew);  // m = -inf gives 0
+          alpha = mf_exp(m - mnew);  // m = -inf gives 0
           float ps = 0.f;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            p[r] = p[r] > PS_NEG_INF ? expf(p[r] - mnew) : 0.f;
+            p[r] = p[r] > PS_NEG_INF ? mf_exp(p[r] - mnew) : 0.f;
             ps += p[r];
           }
           ps += __shfl_xor(ps, 32, 64);
@@ -254,14 +267,16 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
           MfPack b0, b1, b2;
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
+            // p >= 0 cut into three bf16 terms of 8 mantissa bits each
+            // (truncation; both remainders are exact)
             const float pv = p[8 * s + i];
-            const unsigned short h0 = ps_f32_to_bf16(pv);
-            const float r1 = pv - ps_bf16_to_f32(h0);
-            const unsigned short h1 = ps_f32_to_bf16(r1);
-            const float r2 = r1 - ps_bf16_to_f32(h1);
-            b0.u[i] = h0;
-            b1.u[i] = h1;
-            b2.u[i] = ps_f32_to_bf16(r2);
+            const unsigned int h0 = __float_as_uint(pv) & 0xffff0000u;
+            const float r1 = pv - __uint_as_float(h0);
+            const unsigned int h1 = __float_as_uint(r1) & 0xffff0000u;
+            const float r2 = r1 - __uint_as_float(h1);
+            b0.u[i] = (unsigned short)(h0 >> 16);
+            b1.u[i] = (unsigned short)(h1 >> 16);
+            b2.u[i] = (unsigned short)(__float_as_uint(r2) >> 16);
           }
 #pragma unroll
           for (int c = 0; c < CBW; ++c) {
