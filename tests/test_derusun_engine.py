@@ -254,21 +254,22 @@ OTHER_STACKS = [
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("which", range(len(OTHER_STACKS)))
-def test_other_orders_and_sizes(tmp_path, device, which):
+def test_other_orders_and_sizes(tmp_path, device, dtype, which):
     stack, width, vocab, groups, eps, ranks = OTHER_STACKS[which]
     cfg = make_cfg(stack, width=width, vocab=vocab, eps=eps, groups=groups)
     W = make_weights(cfg, seed=40 + which, ranks=ranks)
     path = save_checkpoint(tmp_path / f"o{which}", cfg, W)
     toks = tokens(80, 70 + which, vocab=vocab)
     want = O.forward(cfg, W, toks)
-    eng = make_engine(path, "float32", device)
-    assert rel_err(replay(eng, "a", toks, [None]), want) < 2e-4
-    assert rel_err(replay(eng, "b", toks, [6, 1, 2, 30, 1, 1, None]),
-                   want) < 2e-4
+    eng = make_engine(path, dtype, device)
+    assert close(replay(eng, "a", toks, [None]), want, dtype)
+    assert close(replay(eng, "b", toks, [6, 1, 2, 30, 1, 1, None]), want,
+                 dtype)
     # two requests side by side, cut differently
     half = replay_two(eng, toks, [9, 40, None], [33, 2, None])
-    assert rel_err(half[0], want) < 2e-4 and rel_err(half[1], want) < 2e-4
+    assert close(half[0], want, dtype) and close(half[1], want, dtype)
 
 
 def replay_two(eng, toks, sizes_a, sizes_b):
